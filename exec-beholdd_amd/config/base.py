@@ -115,8 +115,11 @@ def read_config_json(model_dir_or_file: str) -> tuple[dict, str]:
 
 
 def architecture_name(data: dict, origin: str = "config.json") -> str:
-    """The registry tag: `architectures[0]` of config.json."""
+    """The registry tag: `architectures[0]` of config.json, or its `architecture` where the file names its
+    one model class that way."""
     names = data.get("architectures")
+    if names is None and isinstance(data.get("architecture"), str):
+        return data["architecture"]
     if not isinstance(names, list) or len(names) != 1 or not isinstance(names[0], str):
         raise ConfigError(
             f"{origin}: 'architectures' must be a list with exactly one model class name, got {names!r}")

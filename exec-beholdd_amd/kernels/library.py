@@ -161,6 +161,16 @@ class KernelSizes:
                                           i, i, p],
             "bh_kv_order": [i, i],
             "bh_stream_read": [p, ctypes.c_long, i, i, p, p, p],
+            "bh_streams_open": [p, p, i, i, i, p],
+            "bh_streams_rmsnorm": [p, p, p, p, p, i, i, i, i, f, i, p],
+            "bh_streams_update": [p, p, p, p, p, i, i, i, p],
+            "bh_scale": [p, ctypes.c_long, f, p],
+            "bh_relu_squared": [p, i, ctypes.c_long, p],
+            "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, p],
+            "bh_gated_rmsnorm": [p, p, i, i, p, p, i, i, f, i, p],
+            "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, p],
+            "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, p],
+            "bh_rotate_heads": [p, ctypes.c_long, i, i, p, ctypes.c_long, i, i, i, p, i, p, i, i, i, p],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
@@ -735,6 +745,131 @@ class HipKernels(KernelSizes):
             self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
             cos.shape[0] if cos is not None else 0, rot, int(bool(write_kv)), _block_rows(out), self._stream()))
         return True
+
+    # ---- several residual streams, and sublayer results kept apart from the residual ----
+    def streams_open(self, x, out):
+        """out[row, s, :] = x[row, :] for every stream s; x f32 [n, D], out f32 [n, S, D]."""
+        n_rows, streams, width = out.shape
+        if tuple(x.shape) != (n_rows, width):
+            raise KernelError(f"streams_open: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_streams_open(self._ptr(x, "streams_open x", (torch.float32,)),
+                                             self._ptr(out, "streams_open out", (torch.float32,)), n_rows, width, streams,
+                                             self._stream()))
+
+    def streams_rmsnorm(self, x, take, weight, eps, out, rows=None):
+        """out[r] = RMSNorm(sum_s take[s] * x[src, s, :]) * weight with src = rows[r] if rows is given else r;
+        x f32 [*, S, D], take f32 [S] or None (every stream once), weight f32 [D] or None, out [n, D] (rows or
+        `BlockedRows`)."""
+        n_rows, width = out.shape
+        if x.dim() != 3 or x.shape[2] != width or (weight is not None and weight.shape != (width,)) \
+                or (take is not None and take.shape != (x.shape[1],)):
+            raise KernelError(f"streams_rmsnorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
+        if rows is None:
+            if x.shape[0] != n_rows:
+                raise KernelError(f"streams_rmsnorm: {x.shape[0]} input rows for {n_rows} output rows")
+        elif rows.shape != (n_rows,):
+            raise KernelError(f"streams_rmsnorm: {tuple(rows.shape)} row indices for {n_rows} output rows")
+        self._check(self.lib.bh_streams_rmsnorm(
+            self._ptr(x, "streams_rmsnorm x", (torch.float32,)), self._ptr(rows, "streams_rmsnorm rows", (torch.int32,), True),
+            self._ptr(take, "streams_rmsnorm take", (torch.float32,), True),
+            self._ptr(weight, "streams_rmsnorm weight", (torch.float32,), True), self._ptr(out, "streams_rmsnorm out"),
+            _code(out, "streams_rmsnorm out"), n_rows, width, x.shape[1], float(eps), _block_rows(out), self._stream()))
+
+    def streams_update(self, x, y, mix=None, give=None, scale=None):
+        """x[row, t, :] <- sum_s mix[s, t] * x[row, s, :] + give[t] * scale * y[row, :], all streams at once from the
+        old ones; x f32 [n, S, D] in place, y f32 [n, D], mix f32 [S, S] or None (identity), give f32 [S] or None
+        (ones), scale f32 [D] or None."""
+        n_rows, streams, width = x.shape
+        if tuple(y.shape) != (n_rows, width) or (mix is not None and tuple(mix.shape) != (streams, streams)) \
+                or (give is not None and tuple(give.shape) != (streams,)) or (scale is not None and tuple(scale.shape) != (width,)):
+            raise KernelError(f"streams_update: shapes x {tuple(x.shape)}, y {tuple(y.shape)} do not fit")
+        f32 = (torch.float32,)
+        self._check(self.lib.bh_streams_update(
+            self._ptr(x, "streams_update x", f32), self._ptr(y, "streams_update y", f32),
+            self._ptr(mix, "streams_update mix", f32, True), self._ptr(give, "streams_update give", f32, True),
+            self._ptr(scale, "streams_update scale", f32, True), n_rows, width, streams, self._stream()))
+
+    def scale(self, x, factor):
+        """x *= factor, in place; x float32."""
+        self._check(self.lib.bh_scale(self._ptr(x, "scale x", (torch.float32,)), x.numel(), float(factor), self._stream()))
+
+    def relu_squared(self, x):
+        """x <- max(x, 0)^2, in place."""
+        self._check(self.lib.bh_relu_squared(self._ptr(x, "relu_squared x"), _code(x, "relu_squared x"), x.numel(), self._stream()))
+
+    # ---- linear attention with a decay, as a recurrence over a float32 state ----
+    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
+        """For every sequence b of the step (rows seq_start[b] .. seq_start[b + 1] - 1 in order, state row seq_slot[b]) and
+        head h: S <- decay[h] * S + k_t v_t^T, out_t = S^T q_t with q, k, v = silu of the row's slices from q_off, k_off,
+        v_off of `proj` [n, P].  state f32 [slots, H, dim, vdim] in place, out f32 [n, H * vdim]."""
+        n_rows, stride = proj.shape
+        n_seqs = seq_slot.shape[0]
+        if (state.dim() != 4 or tuple(state.shape[1:]) != (n_heads, dim, vdim) or tuple(out.shape) != (n_rows, n_heads * vdim)
+                or tuple(decay.shape) != (n_heads,) or tuple(seq_start.shape) != (n_seqs + 1,)):
+            raise KernelError(f"lightning_scan: shapes proj {tuple(proj.shape)}, state {tuple(state.shape)}, out "
+                              f"{tuple(out.shape)} do not fit {n_heads} heads of {dim} x {vdim} and {n_seqs} sequences")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_lightning_scan(
+            self._ptr(proj, "lightning proj"), _code(proj, "lightning proj"), stride, int(q_off), int(k_off), int(v_off),
+            self._ptr(state, "lightning state", f32), self._ptr(decay, "lightning decay", f32),
+            self._ptr(seq_start, "seq_start", i32), self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "lightning out", f32),
+            n_seqs, n_heads, dim, vdim, self._stream()))
+
+    def gated_rmsnorm(self, o, proj, gate_off, weight, eps, out):
+        """out[r] = RMSNorm(o[r]) * weight * sigmoid(proj[r, gate_off : gate_off + W]); o f32 [n, W], out [n, W] in the
+        type of `proj` (rows or `BlockedRows`)."""
+        n_rows, width = o.shape
+        if tuple(out.shape) != (n_rows, width) or proj.shape[0] != n_rows or gate_off < 0 or gate_off + width > proj.shape[1] \
+                or out.dtype != proj.dtype or (weight is not None and tuple(weight.shape) != (width,)):
+            raise KernelError(f"gated_rmsnorm: shapes o {tuple(o.shape)}, proj {tuple(proj.shape)}, out {tuple(out.shape)} do not fit")
+        gate = self._ptr(proj, "gated_rmsnorm gate") + int(gate_off) * proj.element_size()
+        self._check(self.lib.bh_gated_rmsnorm(
+            self._ptr(o, "gated_rmsnorm o", (torch.float32,)), gate,
+            _code(proj, "gated_rmsnorm gate"), proj.shape[1], self._ptr(weight, "gated_rmsnorm weight", (torch.float32,), True),
+            self._ptr(out, "gated_rmsnorm out"), n_rows, width, float(eps), _block_rows(out), self._stream()))
+
+    # ---- attention over a cached latent ----
+    def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
+                     rank, rot_dim):
+        """From each row of `down` [n, P], at `offset`: c = RMSNorm(rank elements) * weight and the next rot_dim elements
+        rotated (the first `turned` of them, pairs (i, i + turned/2), angle position * freq[i]); key [c | rotated] and
+        value [c | 0] of ONE kv head of size rank + rot_dim go into the cache pages of (sequence, position)."""
+        n_rows = down.shape[0]
+        head = rank + rot_dim
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,) or (weight is not None and tuple(weight.shape) != (rank,)) \
+                or (freq is not None and tuple(freq.shape) != (turned // 2,)):
+            raise KernelError("latent_write: one position and one sequence per row, a weight [rank] and a frequency a pair")
+        self._check_pages(k_pages, v_pages, page_table, 1, head, down.dtype, "latent_write")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_latent_write(
+            self._ptr(down, "latent rows"), _code(down, "latent rows"), down.shape[1], int(offset),
+            self._ptr(weight, "latent norm weight", f32, True), float(eps), self._ptr(freq, "rotation frequencies", f32, True),
+            int(turned), self._ptr(positions, "positions", i32), self._ptr(row_seq, "row_seq", i32),
+            self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"), self._ptr(page_table, "page_table", i32),
+            page_table.shape[1], n_rows, int(rank), int(rot_dim), self.kv_order(k_pages.dtype, head), self._stream()))
+
+    def heads_linear(self, x, x_head, x_first, w, y, y_head, y_first, n_heads):
+        """y[row, h, y_first + o] = sum_i w[h, i, o] * x[row, h, x_first + i]: x [n, >= H * x_head] and y [n, >= H * y_head]
+        are rows of heads of x_head and y_head elements, w [H, n_in, n_out] of their type; float32 sums."""
+        n_rows = x.shape[0]
+        if w.dim() != 3 or w.shape[0] != n_heads or y.shape[0] != n_rows or x.dtype != w.dtype or y.dtype != w.dtype:
+            raise KernelError(f"heads_linear: shapes x {tuple(x.shape)}, w {tuple(w.shape)}, y {tuple(y.shape)} do not fit")
+        self._check(self.lib.bh_heads_linear(
+            self._ptr(x, "heads_linear x"), x.shape[1], int(x_head), int(x_first), self._ptr(w, "heads_linear w"),
+            self._ptr(y, "heads_linear y"), y.shape[1], int(y_head), int(y_first), _code(w, "heads_linear w"), n_rows, n_heads,
+            w.shape[1], w.shape[2], self._stream()))
+
+    def rotate_heads(self, x, x_head, x_first, y, y_head, y_first, freq, turned, positions, n_heads, width):
+        """y[row, h, y_first + i] = x[row, h, x_first + i] for i < width, the first `turned` of them rotated in pairs
+        (i, i + turned/2) by position[row] * freq[i]."""
+        n_rows = x.shape[0]
+        if y.shape[0] != n_rows or positions.shape != (n_rows,) or x.dtype != y.dtype \
+                or (freq is not None and tuple(freq.shape) != (turned // 2,)):
+            raise KernelError(f"rotate_heads: shapes x {tuple(x.shape)}, y {tuple(y.shape)} do not fit")
+        self._check(self.lib.bh_rotate_heads(
+            self._ptr(x, "rotate_heads x"), x.shape[1], int(x_head), int(x_first), self._ptr(y, "rotate_heads y"), y.shape[1],
+            int(y_head), int(y_first), _code(x, "rotate_heads x"), self._ptr(freq, "rotation frequencies", (torch.float32,), True),
+            int(turned), self._ptr(positions, "positions", (torch.int32,)), n_rows, n_heads, int(width), self._stream()))
 
     def stream_read(self, data, workgroups=256, nontemporal=True) -> int:
         """A yardstick, not a product path: read `data` (any contiguous tensor) once the way the streaming kernels

@@ -15,9 +15,11 @@ from ..parts.embedding import Embedding, LMHead
 
 
 class DecoderModel:
-    def __init__(self, config, embedding, blocks, schedule, final_norm, head, shared_parts=()):
+    def __init__(self, config, embedding, blocks, schedule, final_norm, head, shared_parts=(), residual=None):
         self.config = config
         self.embedding, self.blocks, self.final_norm, self.head = embedding, list(blocks), final_norm, head
+        # what turns the embedding's rows into the residual that the blocks update (several streams, say); None: they are it
+        self.residual = residual
         self.shared_parts = list(shared_parts)
         self.schedule = [(int(layer), int(entry)) for layer, entry in schedule]
         for layer, entry in self.schedule:
@@ -50,14 +52,16 @@ class DecoderModel:
         return self.config.max_position
 
     def parts(self):
-        return [self.embedding, *self.shared_parts, *self.blocks, self.final_norm, self.head]
+        opening = [self.residual] if self.residual is not None else []
+        return [self.embedding, *opening, *self.shared_parts, *self.blocks, self.final_norm, self.head]
 
     @property
     def graph_safe(self):
         """True when a decode step of this model may be captured as a HIP graph: every part's
         forward depends on the step's device tensors only."""
         return all(getattr(part, "graph_safe", False)
-                   for part in (self.embedding, *self.blocks, self.final_norm, self.head))
+                   for part in (self.embedding, *self.blocks, self.final_norm, self.head)
+                   ) and (self.residual is None or getattr(self.residual, "graph_safe", False))
 
     @property
     def graph_safe_rows(self) -> int:
@@ -85,6 +89,8 @@ class DecoderModel:
         temporaries are freed before the next one runs; what a block prepares for the next is counted with
         the block that made it), the final norm on the wanted rows and the logits."""
         total = self.embedding.working_bytes(step) if hasattr(self.embedding, "working_bytes") else 0
+        if hasattr(self.residual, "working_bytes"):
+            total += self.residual.working_bytes(step)
         widest = max([block.working_bytes(step) for block in self.blocks if hasattr(block, "working_bytes")], default=0)
         last = 0
         if hasattr(self.final_norm, "working_bytes"):
@@ -105,6 +111,8 @@ class DecoderModel:
         None); `want_rows` (int32 device tensor, may be empty) lists the rows whose logits are
         returned as float32 [len(want_rows), vocab]."""
         hidden = self.embedding.forward(ctx)
+        if self.residual is not None:
+            hidden = self.residual.open(ctx, hidden)
         prepared = None      # the next block's first norm, when the block before could prepare it
         for run, (layer, _entry) in enumerate(self.schedule):
             following = self.blocks[self.schedule[run + 1][0]] if run + 1 < len(self.schedule) else None
@@ -120,14 +128,16 @@ class DecoderModel:
 def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.layers.{}.",
                   embedding_name: str = "model.embed_tokens.weight", final_norm_name: str = "model.norm.weight",
                   head_name: str = "lm_head.weight", final_norm_kind: str = "rmsnorm",
-                  make_embedding=None, make_head=None) -> DecoderModel:
+                  make_embedding=None, make_head=None, make_residual=None) -> DecoderModel:
     """Put a decoder together from the registered parts that `config` names.
 
     `position_encoding` is the registered name of the one encoding that all layers share, or a dictionary
     label -> registered name when layers differ: part builders find them in `shared["position_encodings"][label]`
     (and the one labelled "default", or the first, in `shared["position_encoding"]`).  `make_embedding(config)` and
     `make_head(config, embedding)` replace the plain embedding and head (a scaled embedding, a head that caps
-    its logits); each returns a part with the interface of `parts.embedding`'s."""
+    its logits); each returns a part with the interface of `parts.embedding`'s.  `make_residual(config)` returns a part
+    whose `open(ctx, rows)` turns the embedding's rows into the residual that the blocks update and the final norm
+    reads (several streams: `parts.streams.StreamsResidual`)."""
     shared = {}
     labelled = position_encoding if isinstance(position_encoding, dict) else {"default": position_encoding}
     encodings = {label: POSITION_ENCODINGS.get(name)(config, shared) for label, name in labelled.items()}
@@ -145,4 +155,4 @@ def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.l
     else:
         head = LMHead(config.vocab, config.hidden, head_name)
     return DecoderModel(config, embedding, blocks, config.schedule(), final_norm, head,
-                        shared_parts=list(encodings.values()))
+                        shared_parts=list(encodings.values()), residual=make_residual(config) if make_residual else None)

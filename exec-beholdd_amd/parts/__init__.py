@@ -3,13 +3,18 @@
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, LayerCache,
                    Registry, StepContext)
 from .linear import Linear
-from .norm import RMSNorm
-from .rope import NoPositionEncoding, RotaryEncoding
+from .norm import RMSNorm, ZeroCentredRMSNorm
+from .rope import NoPositionEncoding, RotaryEncoding, RotaryFrequencies
 from .attention import GQAAttention
-from .mlp import SwiGLU
+from .mlp import SquaredReLU, SwiGLU
+from .lightning import LightningAttention
+from .latent_attention import LatentAttention
+from .streams import StreamConnection, StreamMixingBlock, StreamsResidual
 from .block import PreNormBlock
-from .embedding import Embedding, LMHead
+from .embedding import Embedding, LMHead, ScaledLMHead
 
 __all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "CacheNeed", "LayerCache",
            "Registry", "StepContext", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEncoding",
-           "GQAAttention", "SwiGLU", "PreNormBlock", "Embedding", "LMHead"]
+           "GQAAttention", "SwiGLU", "PreNormBlock", "Embedding", "LMHead", "ZeroCentredRMSNorm", "RotaryFrequencies",
+           "SquaredReLU", "LightningAttention", "LatentAttention", "StreamConnection", "StreamMixingBlock", "StreamsResidual",
+           "ScaledLMHead"]

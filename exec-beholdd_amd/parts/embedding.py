@@ -70,3 +70,17 @@ class LMHead:
     def forward(self, ctx, x):
         """x [n, width] -> float32 logits [n, vocab]."""
         return self.linear.forward(ctx, x, out_dtype=torch.float32)
+
+
+class ScaledLMHead(LMHead):
+    """logits = (W x) * scale, the scale applied to the float32 logits."""
+
+    def __init__(self, vocab: int, width: int, name: str | None, scale: float, tied_to: Embedding | None = None):
+        super().__init__(vocab, width, name, tied_to)
+        self.scale = float(scale)
+
+    def forward(self, ctx, x):
+        logits = super().forward(ctx, x)
+        if self.scale != 1.0:
+            ctx.kernels.scale(logits, self.scale)
+        return logits

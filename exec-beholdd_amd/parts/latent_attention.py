@@ -1,0 +1,106 @@
+"""Attention over a cached latent (low-rank keys and values with one rotated key part for all heads).
+
+    q = Wq x                 per head [q_c (dim, not rotated) | q_r (rot_dim, rotated)]
+    Wdkv x = [c_raw | k_r]   c = rms(c_raw) * w_c  (kv_rank),  k_r (rot_dim) rotated, one for all heads
+    k_c = Wuk c,  v = Wuv c  per head (dim and vdim)
+    score_ij = (q_c,i . k_c,j + R_i q_r,i . R_j k_r,j) * scale,  causal softmax,  out = Wo concat_h sum_j p_ij v_j
+
+Only c and k_r are cached.  The up-projections never run over cached positions: since q_c . (Wuk c) = (Wuk^T q_c) . c
+and sum_j p_j (Wuv c_j) = Wuv (sum_j p_j c_j), a head's query is carried into the latent's space and its attended
+latent into the head's values, by one small matrix per head each (`heads_linear`).  What is left in between is the
+paged attention kernels' own case of one key/value head of size kv_rank + rot_dim shared by all query heads, with
+key [c | k_r] and value [c | 0]; prompts and decode steps take the same path, so a position's result does not
+depend on the cut.  The rotation turns the first `rotation.dims` dimensions of the rot_dim part, dimension i with
+i + dims/2, by position * base^(-2i/dims) (angles in float32, no table, no longest position).
+Every size and constant is a constructor parameter.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..weights.binder import TensorSpec
+from .base import MIXERS, CacheNeed
+from .linear import Linear
+from .rope import RotaryFrequencies
+
+
+class LatentAttention:
+    graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None
+    writes_fresh = True    # forward(..., fresh=True) writes its result instead of adding it
+
+    def __init__(self, hidden: int, n_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float,
+                 rotation: RotaryFrequencies, norm_eps: float, prefix: str):
+        if rotation.dims > rot_dim:
+            raise ValueError(f"the rotation turns {rotation.dims} dimensions, the rotated part has {rot_dim}")
+        self.hidden, self.n_heads, self.dim, self.rot_dim = int(hidden), int(n_heads), int(dim), int(rot_dim)
+        self.vdim, self.kv_rank, self.scale = int(vdim), int(kv_rank), float(scale)
+        self.rotation, self.norm_eps, self.prefix = rotation, float(norm_eps), prefix
+        self.q_head = self.dim + self.rot_dim                 # a head of the projected query
+        self.kv_head = self.kv_rank + self.rot_dim            # the one cached key/value head
+        self.down_off = self.n_heads * self.q_head            # where [c_raw | k_r] begins in a projected row
+        self.proj = Linear(hidden, [self.n_heads * self.q_head, self.kv_head], [prefix + "q", prefix + "dkv"])
+        self.out = Linear(self.n_heads * self.vdim, hidden, prefix + "o")
+        self.latent_weight = self.key_up = self.value_up = self.frequencies = None
+
+    @property
+    def input_reader(self):
+        return self.proj.reader()
+
+    def tensor_specs(self):
+        return self.proj.tensor_specs() + self.out.tensor_specs() + [
+            TensorSpec(self.prefix + "dkv.norm", (self.kv_rank,), "norm"),
+            TensorSpec(self.prefix + "uk", (self.n_heads * self.dim, self.kv_rank), "linear"),
+            TensorSpec(self.prefix + "uv", (self.n_heads * self.vdim, self.kv_rank), "linear")]
+
+    def load(self, get):
+        self.proj.load(get)
+        self.out.load(get)
+        self.latent_weight = get(self.prefix + "dkv.norm").to(torch.float32).contiguous()
+        # one matrix per head, [inputs, outputs]: queries go dim -> kv_rank through Wuk as stored, attended latents
+        # kv_rank -> vdim through Wuv transposed
+        self.key_up = get(self.prefix + "uk").view(self.n_heads, self.dim, self.kv_rank).contiguous()
+        self.value_up = get(self.prefix + "uv").view(self.n_heads, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
+        self.frequencies = self.rotation.frequencies(self.latent_weight.device)
+
+    def prepare(self, kernels):
+        self.proj.prepare(kernels)
+        self.out.prepare(kernels)
+
+    def cache_need(self):
+        return CacheNeed(kind="kv", kv_heads=1, head_dim=self.kv_head)
+
+    def working_bytes(self, step) -> int:
+        total = self.proj.working_bytes(step, step.rows) + 2 * step.matrix(step.rows, self.n_heads * self.kv_head)
+        total += step.matrix(step.rows, self.n_heads * self.vdim)
+        if step.sizes is not None:
+            total += step.sizes.attention_working_bytes(step.rows, step.seqs, step.max_rows_per_seq, self.n_heads, 1,
+                                                        self.kv_head, step.max_position, step.act_size)
+        return total + self.out.working_bytes(step, step.rows, accumulate=True)
+
+    def forward(self, ctx, x, hidden, cache, then_norm=None, fresh=False):
+        k = ctx.kernels
+        heads, rank, turned = self.n_heads, self.kv_rank, self.rotation.dims
+        proj = self.proj.forward(ctx, x)
+        if cache.writes:
+            k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, self.frequencies, turned, ctx.positions,
+                           ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table, rank, self.rot_dim)
+        query = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
+        k.heads_linear(proj, self.q_head, 0, self.key_up, query, self.kv_head, 0, heads)
+        k.rotate_heads(proj, self.q_head, self.dim, query, self.kv_head, rank, self.frequencies, turned, ctx.positions,
+                       heads, self.rot_dim)
+        attended = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
+        k.attention(query, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions,
+                    heads, 1, self.kv_head, self.scale, 0, layout=ctx)
+        values = ctx.new_activations(ctx.n_rows, heads * self.vdim)
+        k.heads_linear(attended, self.kv_head, 0, self.value_up, values, self.vdim, 0, heads)
+        self.out.forward(ctx, values, out=hidden, accumulate=not fresh)
+        return None
+
+
+@MIXERS.register("latent_attention")
+def _build_latent_attention(config, layer_index, prefix, shared):
+    sizes = config.layers[layer_index].mixer
+    return LatentAttention(config.hidden, sizes.heads, sizes.dim, sizes.rot_dim, sizes.vdim, sizes.kv_rank, sizes.scale,
+                           RotaryFrequencies(sizes.rot_dims, sizes.rot_base), config.rms_eps, prefix + "mix.")

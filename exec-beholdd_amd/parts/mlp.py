@@ -51,3 +51,50 @@ class SwiGLU:
 @FEED_FORWARDS.register("swiglu")
 def _build_swiglu(config, layer_index, prefix, shared):
     return SwiGLU(config.hidden, config.intermediate, prefix + "mlp.")
+
+
+class SquaredReLU:
+    """Dense feed-forward with one inner matrix: out = Wd relu(Wu x)^2.  Its result is added to `hidden`, or written
+    there when the caller says that `hidden` holds nothing yet (`fresh`)."""
+    graph_safe = True
+    graph_safe_rows = None
+    writes_fresh = True
+
+    def __init__(self, hidden: int, inner: int, prefix: str):
+        self.hidden, self.inner = hidden, inner
+        self.up = Linear(hidden, inner, prefix + "up")
+        self.down = Linear(inner, hidden, prefix + "down")
+
+    @property
+    def input_reader(self):
+        return self.up.reader()
+
+    def tensor_specs(self):
+        return self.up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, get):
+        self.up.load(get)
+        self.down.load(get)
+
+    def prepare(self, kernels):
+        self.up.prepare(kernels)
+        self.down.prepare(kernels)
+
+    def working_bytes(self, step) -> int:
+        return (2 * step.matrix(step.rows, self.inner) + self.up.working_bytes(step, step.rows, accumulate=True)
+                + self.down.working_bytes(step, step.rows, accumulate=True))
+
+    def forward(self, ctx, x, hidden, fresh=False):
+        inner = self.up.forward(ctx, x)
+        ctx.kernels.relu_squared(inner)
+        self.down.forward(ctx, inner, out=hidden, accumulate=not fresh)
+
+
+@FEED_FORWARDS.register("squared_relu")
+def _build_squared_relu(config, layer_index, prefix, shared):
+    return SquaredReLU(config.hidden, config.layers[layer_index].ff, prefix + "mlp.")
+
+
+@FEED_FORWARDS.register("none")
+def _build_no_feed_forward(config, layer_index, prefix, shared):
+    return None

@@ -44,6 +44,37 @@ class RMSNorm:
         return NormRequest(self.weight, self.eps, reader)
 
 
+class ZeroCentredRMSNorm(RMSNorm):
+    """RMSNorm whose stored weight lies around zero: y = x / sqrt(mean(x^2) + eps) * (1 + w).  The sum 1 + w is made
+    once, in float32, when the weight is loaded, and kept in float32 (a bfloat16 could not hold it).  The input is
+    the float32 residual, or several residual streams [n, streams, width] of which the norm reads a weighted sum
+    (`take` [streams] float32; None: every stream once): sum and statistic in float32 in one kernel."""
+
+    reads_streams = True
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.width,), "linear")]      # a random one lies around zero, like a stored one
+
+    def load(self, get):
+        self.weight = (get(self.name).to(torch.float32) + 1.0).contiguous()
+
+    def forward(self, ctx, hidden, rows=None, reader=None, take=None):
+        if hidden.dim() == 2:
+            return super().forward(ctx, hidden, rows=rows, reader=reader)
+        n = hidden.shape[0] if rows is None else rows.shape[0]
+        out = ctx.new_activations(n, self.width, reader=reader)
+        ctx.kernels.streams_rmsnorm(hidden, take, self.weight, self.eps, out, rows=rows)
+        return out
+
+    def request(self, reader=None):
+        raise NotImplementedError("this norm does not ride on the products around it")
+
+
 @NORMS.register("rmsnorm")
 def _build_rmsnorm(config, width, name, shared):
     return RMSNorm(width, config.rms_eps, name)
+
+
+@NORMS.register("rmsnorm_zero_centred")
+def _build_rmsnorm_zero_centred(config, width, name, shared):
+    return ZeroCentredRMSNorm(width, config.rms_eps, name)

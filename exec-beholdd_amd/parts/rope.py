@@ -45,6 +45,26 @@ class RotaryEncoding:
         return self._tables
 
 
+class RotaryFrequencies:
+    """The same rotation without a table: freq[i] = base^(-2i/dims) (computed in float64, kept as float32), and the
+    kernel that rotates forms the angle position * freq[i] as a float32 product and takes its cosine and sine.
+    There is no longest position; `dims` of a vector's dimensions are turned, dimension i with i + dims/2."""
+
+    def __init__(self, dims: int, base: float):
+        if dims <= 0 or dims % 2:
+            raise ValueError(f"rotary width must be positive and even, got {dims}")
+        if not (base > 0.0):
+            raise ValueError(f"rotation base must be positive and finite, got {base}")
+        self.dims, self.base = int(dims), float(base)
+        self._frequencies = None
+
+    def frequencies(self, device) -> torch.Tensor:
+        if self._frequencies is None or self._frequencies.device != torch.device(device):
+            values = np.array([self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)], dtype=np.float64)
+            self._frequencies = torch.from_numpy(values.astype(np.float32)).to(device).contiguous()
+        return self._frequencies
+
+
 class NoPositionEncoding:
     """For mixers whose order information comes from elsewhere (or nowhere)."""
 

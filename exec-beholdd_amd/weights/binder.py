@@ -28,7 +28,7 @@ INT_KINDS = ("I32", "I64")
 class TensorSpec:
     name: str
     shape: tuple
-    init: str = "linear"      # "linear": N(0, std); "norm": 1 + N(0, std); "int": small integers
+    init: str = "linear"      # "linear": N(0, std); "norm": 1 + N(0, std); "identity": I + N(0, std); "int": small integers
     kind: str = "float"       # "float" or "int"
 
 

@@ -4,7 +4,7 @@ The reference has no random-weights mode (its tests hand-write tiny checkpoints,
 crates/beholdd-model/src/qwen3moe/forward.rs:3557-3734).  Each tensor's values depend only
 on (seed, tensor name), so a tensor is the same whatever else the model holds and in
 whatever order tensors are drawn.  Linear and embedding weights are N(0, std); norm weights
-are 1 + N(0, std).
+are 1 + N(0, std), square mixing matrices the identity + N(0, std).
 """
 
 from __future__ import annotations
@@ -35,6 +35,8 @@ def random_tensor(spec: TensorSpec, seed: int, std: float = DEFAULT_STD) -> torc
     values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(std)
     if spec.init == "norm":
         values += np.float32(1.0)
+    elif spec.init == "identity":
+        values += np.eye(*spec.shape, dtype=np.float32)
     return torch.from_numpy(values)
 
 
@@ -49,6 +51,8 @@ def random_tensor_on_device(spec: TensorSpec, seed: int, device, dtype: torch.dt
     values.normal_(0.0, std, generator=generator)
     if spec.init == "norm":
         values += 1.0
+    elif spec.init == "identity":
+        values += torch.eye(*spec.shape, device=device, dtype=dtype)
     return values
 
 

@@ -98,6 +98,103 @@ class TorchKernels:
     def pack_weight(self, w):
         return w
 
+    # ---- residual streams, kept-apart sublayer results ----
+    def streams_open(self, x, out):
+        self.calls.append("streams_open")
+        out.copy_(x.unsqueeze(1).expand_as(out))
+
+    def streams_rmsnorm(self, x, take, weight, eps, out, rows=None):
+        self.calls.append("streams_rmsnorm")
+        src = x if rows is None else x[rows.long()]
+        share = torch.ones(x.shape[1]) if take is None else take.float()
+        u = (src.double() * share.double()[None, :, None]).sum(1).float()
+        y = u * (1.0 / torch.sqrt((u.double() ** 2).mean(-1, keepdim=True) + eps)).float()
+        if weight is not None:
+            y = y * weight.float()
+        out.copy_(y.to(out.dtype))
+
+    def streams_update(self, x, y, mix=None, give=None, scale=None):
+        self.calls.append("streams_update")
+        streams = x.shape[1]
+        m = torch.eye(streams, dtype=torch.float64) if mix is None else mix.double()
+        g = torch.ones(streams, dtype=torch.float64) if give is None else give.double()
+        add = y.double() * (scale.double() if scale is not None else 1.0)
+        new = torch.einsum("st,nsd->ntd", m, x.double()) + g[None, :, None] * add[:, None, :]
+        x.copy_(new.float())
+
+    def scale(self, x, factor):
+        self.calls.append("scale")
+        x.mul_(factor)
+
+    def relu_squared(self, x):
+        self.calls.append("relu_squared")
+        x.copy_((x.float().clamp(min=0) ** 2).to(x.dtype))
+
+    # ---- linear attention with a decay ----
+    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
+        self.calls.append("lightning_scan")
+        silu = lambda z: z / (1 + torch.exp(-z))
+        p = proj.float()
+        for b in range(seq_slot.shape[0]):
+            lo, hi, slot = int(seq_start[b]), int(seq_start[b + 1]), int(seq_slot[b])
+            for row in range(lo, hi):
+                q = silu(p[row, q_off:q_off + n_heads * dim]).reshape(n_heads, dim)
+                k = silu(p[row, k_off:k_off + n_heads * dim]).reshape(n_heads, dim)
+                v = silu(p[row, v_off:v_off + n_heads * vdim]).reshape(n_heads, vdim)
+                s = state[slot] * decay.float()[:, None, None] + k[:, :, None] * v[:, None, :]
+                state[slot] = s
+                out[row] = torch.einsum("hdv,hd->hv", s.double(), q.double()).float().reshape(-1)
+
+    def gated_rmsnorm(self, o, proj, gate_off, weight, eps, out):
+        self.calls.append("gated_rmsnorm")
+        width = o.shape[1]
+        y = o * (1.0 / torch.sqrt((o.double() ** 2).mean(-1, keepdim=True) + eps)).float()
+        if weight is not None:
+            y = y * weight.float()
+        out.copy_((y * torch.sigmoid(proj[:, gate_off:gate_off + width].float())).to(out.dtype))
+
+    # ---- attention over a cached latent ----
+    @staticmethod
+    def _turn(x, freq, turned, positions):
+        """x [n, ..., w]: the first `turned` of the last axis in pairs (i, i + turned/2) by the float32 angle position * freq[i]."""
+        if not turned:
+            return x
+        half = turned // 2
+        angle = (positions.float()[:, None] * freq.float()[None, :]).double()
+        shape = (x.shape[0],) + (1,) * (x.dim() - 2) + (half,)
+        c, s = torch.cos(angle).reshape(shape).float(), torch.sin(angle).reshape(shape).float()
+        a, b, rest = x[..., :half], x[..., half:turned], x[..., turned:]
+        return torch.cat([a * c - b * s, b * c + a * s, rest], dim=-1)
+
+    def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
+                     rank, rot_dim):
+        self.calls.append("latent_write")
+        x = down[:, offset:offset + rank + rot_dim].float()
+        c = x[:, :rank] * (1.0 / torch.sqrt((x[:, :rank].double() ** 2).mean(-1, keepdim=True) + eps)).float()
+        if weight is not None:
+            c = c * weight.float()
+        key = torch.cat([c, self._turn(x[:, rank:], freq, turned, positions)], dim=-1)
+        value = torch.cat([c, torch.zeros(x.shape[0], rot_dim)], dim=-1)
+        for row in range(x.shape[0]):
+            pos = int(positions[row])
+            page = int(page_table[int(row_seq[row]), pos // PAGE])
+            k_pages[page, 0, pos % PAGE, :] = key[row].to(k_pages.dtype)
+            v_pages[page, 0, :, pos % PAGE] = value[row].to(v_pages.dtype)
+
+    def heads_linear(self, x, x_head, x_first, w, y, y_head, y_first, n_heads):
+        self.calls.append("heads_linear")
+        n, n_in, n_out = x.shape[0], w.shape[1], w.shape[2]
+        xs = x[:, :n_heads * x_head].reshape(n, n_heads, x_head)[:, :, x_first:x_first + n_in]
+        result = torch.einsum("nhi,hio->nho", xs.double(), w.double()).float()
+        y[:, :n_heads * y_head].view(n, n_heads, y_head)[:, :, y_first:y_first + n_out] = result.to(y.dtype)
+
+    def rotate_heads(self, x, x_head, x_first, y, y_head, y_first, freq, turned, positions, n_heads, width):
+        self.calls.append("rotate_heads")
+        n = x.shape[0]
+        xs = x[:, :n_heads * x_head].reshape(n, n_heads, x_head)[:, :, x_first:x_first + width].float()
+        y[:, :n_heads * y_head].view(n, n_heads, y_head)[:, :, y_first:y_first + width] = \
+            self._turn(xs, freq, turned, positions).to(y.dtype)
+
     def gemm_swiglu(self, a, w, out):
         self.calls.append("gemm_swiglu")
         both = torch.empty(a.shape[0], w.shape[0], dtype=a.dtype)
