@@ -56,6 +56,10 @@ DEEP = {
                latent(8, 16, 16, 16, 48, 0.5, base=1000.0, ff=96), lightning(4, 32, 48, [0.6, 0.9, 0.99, 0.999], ff=144)],
 }
 CONFIGS = {"mixed": MIXED, "plain": PLAIN, "single": SINGLE, "deep": DEEP}
+# The gain of a configuration's matrices in the tests.  PLAIN has two squared feed-forwards, a sharp attention and no
+# logit scale below one: at unit gain the rounding of bfloat16 activations alone (exact sums, the torch double of
+# the kernels) moves its logits by 3 %, more than the tests allow the kernels.
+GAIN = {"plain": 0.6}
 
 
 def tensor_shapes(config):

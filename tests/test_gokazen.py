@@ -21,7 +21,8 @@ from kernel_emulation import TorchKernels
 def folders(tmp_path_factory):
     made = {}
 
-    def get(name, seed=5, gain=1.0):
+    def get(name, seed=5):
+        gain = gm.GAIN.get(name, 1.0)
         key = (name, seed, gain)
         if key not in made:
             config = gm.CONFIGS[name]

@@ -1,0 +1,388 @@
+"""Gokazen on the GPU: every new kernel alone against the plain implementation's function of the same mechanism, each
+mixer alone through a one-layer model, and the engine over every cut of the work (whole prompts, token by token,
+portions down to two tokens, batches of unequal requests, slots and pages used again) in float32 and bfloat16 on
+configurations that differ in every size, with keys hundreds of positions back and at page borders, long decoding
+through the captured steps, greedy generation through the entry point and the trace replay program."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import gokazen_models as gm
+import plain_gokazen as plain
+import schedules
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOLERANCE = {"float32": 1e-4, "bfloat16": 2e-2}      # max |difference| / max |logit|
+DTYPES = [torch.float32, torch.bfloat16]
+PAGE = 64
+
+
+@pytest.fixture(scope="module")
+def K():
+    from beholdd.kernels import HipKernels
+    return HipKernels("cuda:0")
+
+
+def dev(t):
+    return (torch.from_numpy(np.ascontiguousarray(t)) if isinstance(t, np.ndarray) else t).to("cuda:0")
+
+
+def rel(got, want):
+    got = got.double().cpu().numpy() if isinstance(got, torch.Tensor) else np.asarray(got, np.float64)
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def tol(dtype, f32=2e-5, bf16=1.6e-2):
+    return f32 if dtype == torch.float32 else bf16
+
+
+def rounded(values, dtype):
+    """Random inputs as the kernel's element type holds them, and the same numbers as float32 for the plain side."""
+    t = torch.from_numpy(np.asarray(values, np.float32)).to(dtype)
+    return t, t.to(torch.float32).numpy()
+
+
+# ---- kernels alone ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("rows,streams,width", [(1, 2, 48), (37, 3, 1000), (5, 1, 4100), (70, 16, 260), (3, 4, 9000)])
+def test_streams_kernels(K, rows, streams, width):
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, width)).astype(np.float32)
+    opened = torch.empty(rows, streams, width, device="cuda:0")
+    K.streams_open(dev(x), opened)
+    assert torch.equal(opened.cpu(), torch.from_numpy(x)[:, None, :].expand(rows, streams, width))
+    old = rng.standard_normal((rows, streams, width)).astype(np.float32)
+    y = rng.standard_normal((rows, width)).astype(np.float32)
+    names = {"c.mix": rng.standard_normal((streams, streams)).astype(np.float32), "c.out": rng.standard_normal(streams).astype(np.float32)}
+    scale = rng.standard_normal(width).astype(np.float32)
+    want = np.stack(plain.mix_streams([old[:, s] for s in range(streams)], names, "c.", y * scale), axis=1)
+    state = dev(old.copy())
+    K.streams_update(state, dev(y), dev(names["c.mix"]), dev(names["c.out"]), dev(scale))
+    assert rel(state, want) < 2e-6
+    state = dev(old.copy())             # nothing given: every stream keeps itself and takes y once
+    K.streams_update(state, dev(y))
+    assert rel(state, old + y[:, None, :]) < 1e-6
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("rows,streams,width,eps", [(1, 2, 48, 1e-6), (33, 3, 1000, 1e-5), (4, 1, 5120, 1e-6), (70, 5, 260, 1e-2),
+                                                    (3, 2, 9001, 1e-6)])
+def test_streams_rmsnorm(K, out_dtype, rows, streams, width, eps):
+    rng = np.random.default_rng(width)
+    x = rng.standard_normal((2 * rows, streams, width)).astype(np.float32) * 3
+    take = rng.standard_normal(streams).astype(np.float32)
+    w = (0.3 * rng.standard_normal(width)).astype(np.float32)
+    picked = rng.permutation(2 * rows)[:rows].astype(np.int32)
+    u = sum(np.float64(take[s]) * x[:, s].astype(np.float64) for s in range(streams)).astype(np.float32)
+    want = plain.zero_centred_norm(u, w, eps)
+    out = torch.empty(2 * rows, width, dtype=out_dtype, device="cuda:0")
+    K.streams_rmsnorm(dev(x), dev(take), dev(1 + w), eps, out)
+    assert rel(out, want) < tol(out_dtype, bf16=8e-3)
+    out = torch.empty(rows, width, dtype=out_dtype, device="cuda:0")       # chosen rows, every stream once
+    K.streams_rmsnorm(dev(x), None, dev(1 + w), eps, out, rows=dev(picked))
+    assert rel(out, plain.zero_centred_norm(x.astype(np.float64).sum(1).astype(np.float32)[picked], w, eps)) < tol(out_dtype, bf16=8e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_small_elementwise_kernels(K, dtype):
+    rng = np.random.default_rng(0)
+    t, x = rounded(rng.standard_normal((7, 333)) * 4, dtype)
+    on_device = dev(t)
+    K.relu_squared(on_device)
+    assert rel(on_device, plain.squared_relu(x)) < tol(dtype, bf16=4e-3)
+    logits = dev(rng.standard_normal((5, 77)).astype(np.float32))
+    before = logits.cpu().numpy()
+    K.scale(logits, 0.3)
+    assert rel(logits, before * np.float32(0.3)) < 1e-7
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim,vdim,decay,lengths", [
+    (2, 16, 24, [0.9, 0.999], [5, 1, 40]),             # key and value sizes differ, a value tile that is not full
+    (1, 64, 64, [0.97], [130]),                         # one head, several stages of rows
+    (4, 8, 8, [0.5, 0.8, 0.95, 1.0], [3, 17]),          # small heads, a head that forgets nothing
+    (3, 20, 12, [0.99, 0.9, 0.7], [33, 2, 2, 16]),      # sizes that are no power of two
+    (2, 128, 128, [0.99, 0.95], [70]),                  # the sizes of a large model's heads: two value tiles
+    (1, 200, 72, [0.98], [19]),                         # a key size whose slices are padded
+])
+def test_lightning_scan(K, dtype, heads, dim, vdim, decay, lengths):
+    """The recurrence over ragged rows of several sequences, into slots in another order than the batch's, and then
+    continued by a second call from the state the first one left (one row a sequence, as in decoding)."""
+    rng = np.random.default_rng(dim * vdim)
+    keys, values = heads * dim, heads * vdim
+    stride, q_off, k_off, v_off = 2 * keys + 2 * values + 5, 3, 3 + keys, 3 + 2 * keys      # slices at odd places of a wider row
+    slots = list(rng.permutation(len(lengths) + 2)[:len(lengths)])
+    state = torch.zeros(len(lengths) + 2, heads, dim, vdim, device="cuda:0")
+    untouched = [s for s in range(len(lengths) + 2) if s not in slots]
+    state[untouched] = 7.0
+    kept = {}
+    for lengths_now in (lengths, [1] * len(lengths)):
+        n = sum(lengths_now)
+        t, proj = rounded(rng.standard_normal((n, stride)), dtype)
+        starts = np.concatenate([[0], np.cumsum(lengths_now)]).astype(np.int32)
+        out = torch.empty(n, values, device="cuda:0")
+        K.lightning_scan(dev(t), q_off, k_off, v_off, state, dev(np.asarray(decay, np.float32)), dev(starts),
+                         dev(np.asarray(slots, np.int32)), out, heads, dim, vdim)
+        for b, slot in enumerate(slots):
+            rows = proj[starts[b]:starts[b + 1]]
+            q = plain.silu(rows[:, q_off:q_off + keys]).reshape(-1, heads, dim).astype(np.float64)
+            k = plain.silu(rows[:, k_off:k_off + keys]).reshape(-1, heads, dim).astype(np.float64)
+            v = plain.silu(rows[:, v_off:v_off + values]).reshape(-1, heads, vdim).astype(np.float64)
+            s = kept.get(slot, np.zeros((heads, dim, vdim)))
+            want = np.zeros((len(rows), heads, vdim))
+            for i in range(len(rows)):
+                s = np.asarray(decay)[:, None, None] * s + k[i][:, :, None] * v[i][:, None, :]
+                want[i] = np.einsum("hdv,hd->hv", s, q[i])
+            kept[slot] = s
+            assert rel(out[starts[b]:starts[b + 1]], want.reshape(len(rows), -1)) < 3e-5, (b, lengths_now)
+            assert rel(state[slot], s) < 3e-5
+        assert bool((state[untouched] == 7.0).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width,eps", [(1, 48, 1e-6), (9, 512, 1e-5), (40, 3000, 1e-6)])
+def test_gated_rmsnorm(K, dtype, rows, width, eps):
+    rng = np.random.default_rng(rows)
+    o = (rng.standard_normal((rows, width)) * 5).astype(np.float32)
+    t, proj = rounded(rng.standard_normal((rows, width + 11)) * 2, dtype)
+    w = (1 + 0.3 * rng.standard_normal(width)).astype(np.float32)
+    out = torch.empty(rows, width, dtype=dtype, device="cuda:0")
+    K.gated_rmsnorm(dev(o), dev(t), 11, dev(w), eps, out)
+    want = plain.plain_weight_norm(o, w, eps).astype(np.float64) * plain.sigmoid(proj[:, 11:])
+    assert rel(out, want) < tol(dtype, bf16=8e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,heads,n_in,n_out", [(1, 3, 16, 48), (37, 2, 24, 40), (16, 8, 128, 300), (130, 1, 7, 5)])
+def test_heads_linear(K, dtype, rows, heads, n_in, n_out):
+    rng = np.random.default_rng(n_in)
+    x_head, y_head, x_first, y_first = n_in + 6, n_out + 3, 4, 2
+    tx, x = rounded(rng.standard_normal((rows, heads * x_head + 1)), dtype)
+    tw, w = rounded(rng.standard_normal((heads, n_in, n_out)) / np.sqrt(n_in), dtype)
+    y = torch.full((rows, heads * y_head), 9.0, dtype=dtype, device="cuda:0")
+    K.heads_linear(dev(tx), x_head, x_first, dev(tw), y, y_head, y_first, heads)
+    got = y.float().cpu().numpy().reshape(rows, heads, y_head)
+    for head in range(heads):
+        want = plain.linear(x[:, head * x_head + x_first:head * x_head + x_first + n_in], w[head].T)
+        assert rel(got[:, head, y_first:y_first + n_out], want) < tol(dtype, bf16=8e-3)
+    assert (got[:, :, :y_first] == 9.0).all() and (got[:, :, y_first + n_out:] == 9.0).all()        # nothing else is written
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,turned,base", [(16, 16, 10000.0), (16, 8, 500.0), (6, 4, 50.0), (64, 64, 20000.0)])
+def test_rotate_heads(K, dtype, width, turned, base):
+    from beholdd.parts import RotaryFrequencies
+    rng = np.random.default_rng(width)
+    rows, heads = 21, 3
+    positions = np.array(sorted(rng.integers(0, 5000, size=rows)), np.int32)
+    positions[0], positions[-1] = 0, 100000
+    tx, x = rounded(rng.standard_normal((rows, heads * (width + 5))), dtype)
+    y = torch.zeros(rows, heads * (width + 2), dtype=dtype, device="cuda:0")
+    freq = RotaryFrequencies(turned, base).frequencies("cuda:0")
+    K.rotate_heads(dev(tx), width + 5, 5, y, width + 2, 1, freq, turned, dev(positions), heads, width)
+    want = plain.rotate(x.reshape(rows, heads, width + 5)[:, :, 5:], positions, turned, base)
+    got = y.float().cpu().numpy().reshape(rows, heads, width + 2)
+    assert rel(got[:, :, 1:1 + width], want) < tol(dtype, f32=3e-5, bf16=8e-3)
+
+
+# ---- every mixer alone, through the engine, as a model of one layer ---------------------------------------------
+
+ALONE = {
+    "lightning": {"architecture": "Gokazen", "vocab": 61, "width": 40, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+                  "layers": [gm.lightning(3, 24, 40, [0.9, 0.99, 0.999])]},
+    "latent": {"architecture": "Gokazen", "vocab": 61, "width": 40, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+               "layers": [gm.latent(5, 24, 8, 40, 56, 0.8, base=300.0)]},
+    "latent, half turned": {"architecture": "Gokazen", "vocab": 61, "width": 40, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+                            "layers": [gm.latent(2, 8, 24, 16, 72, 1.1, base=1e5, dims=12)]},
+    "feed-forward": {"architecture": "Gokazen", "vocab": 61, "width": 40, "streams": 2, "logit_scale": 2.0, "norm": {"eps": 1e-5},
+                     "layers": [gm.lightning(1, 4, 4, [0.5], ff=100)]},
+}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, seed=5):
+        if (name, seed) not in made:
+            config = gm.CONFIGS.get(name) or ALONE[name]
+            # (the feed-forward squares its inner values: at unit gain its bfloat16 rounding alone is the tolerance)
+            gain = 0.5 if name == "feed-forward" else gm.GAIN.get(name, 1.0)
+            folder = gm.write_model(tmp_path_factory.mktemp("gokazen"), config, gm.random_weights(config, seed, gain))
+            made[(name, seed)] = (folder, *plain.load(folder))
+        return made[(name, seed)]
+
+    return get
+
+
+def engine_for(folder, dtype, max_tokens=4096, **kw):
+    from beholdd.engine import Engine
+    return Engine(folder, dtype=dtype, max_tokens=max_tokens, **kw)
+
+
+def check(label, got, want, tolerance):
+    for index, (g, e) in enumerate(zip(got, want)):
+        assert g.shape == e.shape, (label, index, g.shape, e.shape)
+        assert np.isfinite(g).all(), (label, index)
+        error = schedules.relative_error(g, e)
+        if error >= tolerance:
+            per_row = np.abs(g.astype(np.float64) - e).max(axis=1) / np.abs(e).max()
+            pytest.fail(f"{label}: request {index} (length {len(g)}): error {error:.3e} >= {tolerance}; "
+                        f"first wrong position {int(np.argmax(per_row >= tolerance))}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ALONE))
+def test_every_mixer_alone(folders, name, dtype):
+    folder, config, weights = folders(name)
+    requests = schedules.random_requests(config["vocab"], [1, 2, 63, 64, 65, 130, 200], seed=2)
+    want = [plain.forward(config, weights, r) for r in requests]
+    engine = engine_for(folder, dtype)
+    check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
+    check("one by one", schedules.tail_one_by_one(engine, requests, tail=70), want, TOLERANCE[dtype])
+    check("portions", schedules.portions(engine, requests), want, TOLERANCE[dtype])
+
+
+# ---- the engine over every cut ------------------------------------------------------------------------------------
+
+LENGTHS = {"mixed": [5, 11, 1, 70, 33, 128, 300], "plain": [1, 7, 23, 64, 90, 200], "single": [3, 65, 130, 2, 31],
+           "deep": [2, 50, 129, 260]}
+
+
+@pytest.fixture(scope="module")
+def expected(folders):
+    cache = {}
+
+    def get(name):
+        if name not in cache:
+            folder, config, weights = folders(name)
+            requests = schedules.random_requests(config["vocab"], LENGTHS[name], seed=11)
+            cache[name] = (folder, requests, [plain.forward(config, weights, r) for r in requests])
+        return cache[name]
+
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(LENGTHS))
+def test_every_cut_matches_the_plain_implementation(expected, name, dtype):
+    folder, requests, want = expected(name)
+    engine = engine_for(folder, dtype)
+    tolerance = TOLERANCE[dtype]
+    whole = schedules.whole(engine, requests)
+    check("whole", whole, want, tolerance)
+    tail = schedules.tail_one_by_one(engine, requests, tail=32)
+    check("last 32 one by one", tail, want, tolerance)
+    for batch_size in (3, len(requests)):
+        batched = schedules.batches(engine, requests, batch_size=batch_size)
+        check(f"batches of {batch_size}", batched, want, tolerance)
+    in_portions = schedules.portions(engine, requests)
+    check("portions", in_portions, want, tolerance)
+    pairs = schedules.portions(engine, requests, sizes=(2, 2, 3, 2, 1, 2), rest_every=3)
+    check("portions of two and three", pairs, want, tolerance)
+    check("tail vs whole", tail, whole, tolerance / 2)
+    check("batches vs whole", batched, whole, tolerance / 2)
+    check("portions vs whole", in_portions, whole, tolerance / 2)
+    engine.cache.check_invariants()
+    assert engine.cache.live_slots() == [] and engine.cache.free_page_count() == engine.cache.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_changes_nothing_for_its_members(expected, dtype):
+    """Float32 rows do not depend on their batch at all; bfloat16 ones within rounding (other kernels by row count)."""
+    folder, requests, _ = expected("mixed")
+    engine = engine_for(folder, dtype)
+    alone = schedules.whole(engine, requests)
+    from beholdd.engine import StepEntry
+    slots = [engine.alloc_slot() for _ in requests]
+    together = engine.step([StepEntry(s, r, list(range(len(r)))) for s, r in zip(slots, requests)]).float().cpu().numpy()
+    at = 0
+    for r, a in zip(requests, alone):
+        error = schedules.relative_error(together[at:at + len(r)], a)
+        assert error < (1e-6 if dtype == "float32" else 1e-2), error
+        at += len(r)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_far_keys_and_long_decoding(folders, dtype):
+    """A request of 700 tokens whose far tokens decide its logits (test_gokazen.py shows that they do): the prompt in
+    portions that end at, before and after page borders, then 150 tokens one by one through the captured steps, in a
+    cache whose pages were used before by other requests."""
+    folder, config, weights = folders("deep")
+    long_one = schedules.random_requests(config["vocab"], [700], seed=31)[0]
+    want = plain.forward(config, weights, long_one)
+    engine = engine_for(folder, dtype, max_tokens=1024)
+    schedules.whole(engine, schedules.random_requests(config["vocab"], [300, 90], seed=32))      # pages and slots that are used again
+    from beholdd.engine import StepEntry
+    slot = engine.alloc_slot()
+    rows, at = [], 0
+    for size in (63, 1, 64, 65, 127, 2, 100, 128):
+        rows.append(engine.step([StepEntry(slot, long_one[at:at + size], list(range(size)))]).float().cpu().numpy())
+        at += size
+    assert at == 550
+    for token in long_one[at:]:
+        rows.append(engine.step([StepEntry(slot, [token], [0])]).float().cpu().numpy().copy())
+    engine.free_slot(slot)
+    check("long", [np.concatenate(rows)], [want], TOLERANCE[dtype])
+    if engine.graphs is not None:
+        assert len(engine.graphs.graphs) >= 1          # the one-token steps were captured and replayed
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, dtype):
+    import beholdd
+    folder, config, weights = folders("mixed")
+    prompts = schedules.random_requests(config["vocab"], [1, 9, 30, 70], seed=6)
+    max_new = [12, 9, 12, 40]
+    engine = beholdd.Engine(folder, dtype=dtype, max_tokens=1024)
+    results = engine.generate(prompts, max_new_tokens=max_new)
+    assert len({token for r in results for token in r.token_ids}) >= 6
+    for prompt, result, n in zip(prompts, results, max_new):
+        if dtype == "float32":
+            assert result.token_ids == plain.greedy(config, weights, prompt, n)
+            continue
+        fed = list(prompt)
+        for token in result.token_ids:          # as good as the plain choice within rounding
+            row = plain.forward(config, weights, fed)[-1]
+            assert row[token] >= row.max() - 3e-2 * np.abs(row).max(), (fed, token)
+            fed.append(token)
+    sampled = engine.generate(prompts, max_new_tokens=8, temperature=0.9, top_k=20, top_p=0.9, seed=4)
+    again = engine.generate(prompts, max_new_tokens=8, temperature=0.9, top_k=20, top_p=0.9, seed=4)
+    assert [r.token_ids for r in sampled] == [r.token_ids for r in again]
+    engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_and_generate_programs(folders, tmp_path, dtype):
+    folder, config, weights = folders("single")
+    requests = schedules.random_requests(config["vocab"], [40, 7, 66], seed=9)
+    want = [plain.forward(config, weights, r) for r in requests]
+    steps = schedules.trace_of(schedules.batches, requests, batch_size=3)
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                          "--out", str(tmp_path / "out"), "--max-tokens", "256"],
+                         input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    done = {f"r{i}": 0 for i in range(len(requests))}
+    for record in steps:
+        got = np.fromfile(tmp_path / "out" / f"{record['step']}.f32", dtype="<f4").reshape(-1, config["vocab"])
+        rows = []
+        for entry in record["entries"]:
+            index = int(entry["id"][1:])
+            rows.append(want[index][[done[entry["id"]] + w for w in entry["want"]]])
+            done[entry["id"]] += len(entry["tokens"])
+        assert schedules.relative_error(got, np.concatenate(rows)) < TOLERANCE[dtype], record["step"]
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "beholdd"), "generate", "--model", folder, "--dtype", dtype,
+                          "--prompt-ids", ",".join(str(t) for t in requests[1]), "--max-new-tokens", "5"],
+                         capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    if dtype == "float32":
+        expected_tokens = plain.greedy(config, weights, requests[1], 5)
+        assert all(str(token) in run.stdout for token in expected_tokens), (run.stdout, expected_tokens)
