@@ -53,6 +53,11 @@ def parse():
                              "128 tokens each at temperature 1) and print its tokens per second")
     parser.add_argument("--hbm-ceiling", action="store_true",
                         help="measure what a plain streaming read and a copy of 8 GB reach on this GPU, print it and exit")
+    parser.add_argument("--gokazen", action="store_true",
+                        help="the Gokazen design (linear attention with a decay, attention over a cached latent, residual "
+                             "streams) at layer sizes of real models beside Qwen3 at equal width and depth: prefill and decode "
+                             "tokens per second of both, and every kernel of the new design beside its like with the fraction "
+                             "of its roofline; prints one JSON line and exits")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
                              "top-k, with top-p on rows of three spreads, with both), print the microseconds and exit")
@@ -227,6 +232,176 @@ def sampling_times(torch):
     return out
 
 
+# ---- the Gokazen design beside Qwen3 at equal width and depth ---------------------------------------------
+
+def gokazen_config(width, heads, layers, ff, vocab, rank=192, rot=64):
+    """`layers` layers, three with linear attention to every one with attention over a cached latent (heads of 128, a
+    latent of `rank` and a shared rotated key part of `rot`), two residual streams, a dense feed-forward in every layer."""
+    decay = [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(heads - 1, 1)) for h in range(heads)]
+    lightning = {"type": "lightning", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "decay": decay},
+                 "mlp": {"kind": "dense", "ff": ff}}
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+              "mixer": {"heads": heads, "dim": 128, "rot_dim": rot, "vdim": 128, "kv_rank": rank, "scale": (128 + rot) ** -0.5,
+                        "rot": {"base": 10000.0, "dims": rot}}}
+    return {"architecture": "Gokazen", "vocab": vocab, "width": width, "streams": 2, "logit_scale": 1.0, "norm": {"eps": 1e-6},
+            "layers": [latent if i % 4 == 3 else lightning for i in range(layers)]}
+
+
+def timed(call, torch, repeats=20):
+    """Median microseconds of `call()` on the device (two calls first, untimed)."""
+    call(), call()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(repeats):
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        call()
+        end.record()
+        end.synchronize()
+        times.append(begin.elapsed_time(end) * 1e3)
+    return sorted(times)[len(times) // 2]
+
+
+def gokazen_kernels(K, torch, width, heads, rank, rot, context, streams=2):
+    """Every kernel of the new design and its like among Qwen3's, alone, at a prompt of 2,048 rows and at a decode step of 8
+    rows over `context` cached tokens: microseconds and the fraction of the roofline (the slower of its bytes at the HBM
+    peak and its operations at the peak of the units it runs on: FMA for the recurrence, matrix cores for what is a
+    matrix product)."""
+    from types import SimpleNamespace
+    bf16, f32, dev = torch.bfloat16, torch.float32, "cuda:0"
+    dim = vdim = 128
+    page = K.page_size
+    out = {}
+
+    def note(name, us, n_bytes, flops=0.0, peak=PEAK_FLOPS["fp32"]):
+        floor = max(n_bytes / (PEAK_HBM_GBS * 1e9), flops / peak) * 1e6
+        out[name] = {"us": round(us, 1), "roofline_us": round(floor, 2), "fraction": round(floor / us, 3)}
+
+    def pages_for(n_seqs, length, kv_heads, head):
+        per = -(-length // page)
+        k_pages = torch.randn(n_seqs * per, kv_heads, page, head, device=dev).to(bf16)
+        v_pages = torch.randn(n_seqs * per, kv_heads, head, page, device=dev).to(bf16)
+        table = torch.arange(n_seqs * per, dtype=torch.int32, device=dev).view(n_seqs, per).contiguous()
+        return k_pages, v_pages, table
+
+    for rows, seqs, past, tag in ((2048, 1, 0, "prompt of 2,048"), (8, 8, context - 1, f"decode of 8 at {context}")):
+        each = rows // seqs
+        starts = torch.arange(0, rows + 1, each, dtype=torch.int32, device=dev)
+        slots = torch.arange(seqs, dtype=torch.int32, device=dev)
+        positions = (torch.arange(rows, dtype=torch.int32, device=dev) % each + past).contiguous()
+        row_seq = (torch.arange(rows, dtype=torch.int32, device=dev) // each).contiguous()
+        layout = SimpleNamespace(seq_start=starts, n_seqs=seqs, max_rows_per_seq=each, max_position=past + each - 1)
+        # -- the new design
+        proj = torch.randn(rows, 4 * heads * dim, device=dev).to(bf16)
+        state = torch.zeros(seqs, heads, dim, vdim, device=dev)
+        decay = torch.full((heads,), 0.99, device=dev)
+        mixed = torch.empty(rows, heads * vdim, device=dev)
+        us = timed(lambda: K.lightning_scan(proj, 0, heads * dim, 2 * heads * dim, state, decay, starts, slots, mixed, heads, dim, vdim), torch)
+        note(f"lightning_scan, {tag}", us, 2 * state.numel() * 4 + rows * 3 * heads * dim * 2 + mixed.numel() * 4, 4.0 * rows * heads * dim * vdim)
+        gated = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        weight = torch.ones(heads * vdim, device=dev)
+        us = timed(lambda: K.gated_rmsnorm(mixed, proj, 3 * heads * dim, weight, 1e-6, gated), torch)
+        note(f"gated_rmsnorm, {tag}", us, mixed.numel() * 4 + 2 * gated.numel() * 2)
+        x = torch.randn(rows, streams, width, device=dev)
+        normed = torch.empty(rows, width, device=dev, dtype=bf16)
+        take, ones = torch.ones(streams, device=dev), torch.ones(width, device=dev)
+        us = timed(lambda: K.streams_rmsnorm(x, take, ones, 1e-6, normed), torch)
+        note(f"streams_rmsnorm, {tag}", us, x.numel() * 4 + normed.numel() * 2)
+        y, mix = torch.randn(rows, width, device=dev), torch.eye(streams, device=dev)
+        us = timed(lambda: K.streams_update(x, y, mix, take, ones), torch)
+        note(f"streams_update, {tag}", us, 2 * x.numel() * 4 + y.numel() * 4)
+        q_head, kv_head = dim + rot, rank + rot
+        qd = torch.randn(rows, heads * q_head + kv_head, device=dev).to(bf16)
+        k_pages, v_pages, table = pages_for(seqs, past + each, 1, kv_head)
+        freq, latent_weight = torch.ones(rot // 2, device=dev), torch.ones(rank, device=dev)
+        us = timed(lambda: K.latent_write(qd, heads * q_head, latent_weight, 1e-6, freq, rot, positions, row_seq,
+                                          k_pages, v_pages, table, rank, rot), torch)
+        note(f"latent_write, {tag}", us, rows * kv_head * 2 * 3)
+        key_up = torch.randn(heads, dim, rank, device=dev).to(bf16)
+        query = torch.empty(rows, heads * kv_head, device=dev, dtype=bf16)
+        us = timed(lambda: K.heads_linear(qd, q_head, 0, key_up, query, kv_head, 0, heads), torch)
+        note(f"heads_linear (queries into the latent), {tag}", us, key_up.numel() * 2 + rows * heads * (dim + rank) * 2,
+             2.0 * rows * heads * dim * rank, PEAK_FLOPS["bf16"])
+        us = timed(lambda: K.rotate_heads(qd, q_head, dim, query, kv_head, rank, freq, rot, positions, heads, rot), torch)
+        note(f"rotate_heads, {tag}", us, 2 * rows * heads * rot * 2)
+        attended = torch.empty_like(query)
+        scale = (dim + rot) ** -0.5
+        us = timed(lambda: K.attention(query, attended, k_pages, v_pages, table, row_seq, positions, heads, 1, kv_head, scale, 0, layout=layout), torch)
+        keys_seen = seqs * (past + each) if each == 1 else each * (each + 1) // 2
+        note(f"attention over the latent ({heads} heads on one of {kv_head}), {tag}", us,
+             2 * seqs * (past + each) * kv_head * 2 + 2 * query.numel() * 2, 4.0 * keys_seen * heads * kv_head, PEAK_FLOPS["bf16"])
+        value_up = torch.randn(heads, rank, vdim, device=dev).to(bf16)
+        values = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        us = timed(lambda: K.heads_linear(attended, kv_head, 0, value_up, values, vdim, 0, heads), torch)
+        note(f"heads_linear (latents into values), {tag}", us, value_up.numel() * 2 + rows * heads * (rank + vdim) * 2,
+             2.0 * rows * heads * rank * vdim, PEAK_FLOPS["bf16"])
+        inner = torch.randn(rows, 3 * width, device=dev).to(bf16)
+        us = timed(lambda: K.relu_squared(inner), torch)
+        note(f"relu_squared, {tag}", us, 2 * inner.numel() * 2)
+        # -- their like in Qwen3 at the same width: 4 query heads of 128 to a kv head
+        kv_heads = max(heads // 4, 1)
+        hidden = torch.randn(rows, width, device=dev)
+        us = timed(lambda: K.rmsnorm(hidden, ones, 1e-6, normed), torch)
+        note(f"qwen3 rmsnorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        qkv = torch.randn(rows, (heads + 2 * kv_heads) * dim, device=dev).to(bf16)
+        gk, gv, gtable = pages_for(seqs, past + each, kv_heads, dim)
+        q_out = torch.empty(rows, heads * dim, device=dev, dtype=bf16)
+        head_weight = torch.ones(dim, device=dev)
+        cos = torch.ones(past + each, dim // 2, device=dev)
+        us = timed(lambda: K.qk_norm_rope_cache(qkv, q_out, head_weight, head_weight, 1e-6, cos, cos, positions, row_seq, gk, gv,
+                                                gtable, heads, kv_heads, dim, True, past + each - 1), torch)
+        note(f"qwen3 qk_norm_rope_cache, {tag}", us, 2 * qkv.numel() * 2)
+        g_out = torch.empty_like(q_out)
+        us = timed(lambda: K.attention(q_out, g_out, gk, gv, gtable, row_seq, positions, heads, kv_heads, dim, dim ** -0.5, 0, layout=layout), torch)
+        note(f"qwen3 attention ({heads} heads on {kv_heads} of {dim}), {tag}", us,
+             2 * seqs * (past + each) * kv_heads * dim * 2 + 2 * q_out.numel() * 2, 4.0 * keys_seen * heads * dim, PEAK_FLOPS["bf16"])
+        gate_up = torch.randn(rows, 6 * width, device=dev).to(bf16)
+        activated = torch.empty(rows, 3 * width, device=dev, dtype=bf16)
+        us = timed(lambda: K.swiglu(gate_up, activated), torch)
+        note(f"qwen3 swiglu, {tag}", us, 3 * activated.numel() * 2)
+    return out
+
+
+def gokazen_bench(args, torch):
+    from beholdd.engine import Engine, random_model_on_device
+
+    device, points = "cuda:0", []
+    t = min(args.prefill_tokens, args.context)
+    layers = args.layers or 8
+    for width, heads in ((2048, 16), (4096, 32)):
+        pair = {"gokazen": gokazen_config(width, heads, layers, 3 * width, 32768),
+                "qwen3": dict(QWEN3_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
+                              num_key_value_heads=heads // 4, intermediate_size=3 * width, vocab_size=32768)}
+        point = {"width": width, "heads": heads, "layers": layers}
+        for name, config in pair.items():
+            model = random_model_on_device(config, seed=0, dtype="bfloat16", device=device)
+            engine = Engine(model=model, dtype="bfloat16", max_tokens=args.batch * (-(-args.context // 64) * 64),
+                            max_slots=args.batch, device=device)
+            parameters = sum(int(np_prod(spec.shape)) for spec in model.tensor_specs())
+            seconds, _ = decode_run(engine, args.batch, args.context, args.steps, args.warmup, torch)
+            prefill = prefill_run(engine, t, torch)
+            point[name] = {"parameters": parameters, "decode_ms_per_step": round(seconds * 1e3, 4),
+                           "decode_tok_per_s": round(args.batch / seconds, 1), "prefill_ms": round(prefill * 1e3, 3),
+                           "prefill_tok_per_s": round(t / prefill, 1)}
+            kernels = engine.kernels
+            del engine, model
+            torch.cuda.empty_cache()
+        points.append(point)
+    line = {"metric": f"Gokazen beside Qwen3 at equal width and depth: decode tok/s @ batch {args.batch}, context {args.context}; prefill of {t} tokens",
+            "unit": "tok/s", "value": points[-1]["gokazen"]["decode_tok_per_s"], "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "points": points,
+            "kernels": gokazen_kernels(kernels, torch, 4096, 32, 192, 64, args.context)}
+    print(json.dumps(line))
+    return 0
+
+
+def np_prod(shape):
+    total = 1
+    for axis in shape:
+        total *= int(axis)
+    return total
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -239,6 +414,8 @@ def main():
     if args.sampling:
         print(json.dumps(sampling_times(torch)))
         return 0
+    if args.gokazen:
+        return gokazen_bench(args, torch)
 
     from beholdd.engine import Engine, random_model_on_device
 

@@ -734,18 +734,18 @@ extern "C" int bh_qk_norm_rope_cache_sums(const float* sums, int parts, void* q_
 // at a time: scores (one thread per key), running maximum and sum in float32 (online softmax),
 // then the value sum with threads spread over (key subset, dimension).
 
-#define AG_THREADS 256
+#define AG_THREADS 256   // threads of a workgroup for heads up to that size; wider heads take 512 or 1024 (a thread per dimension)
 
-template <typename T>
-__global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window, int kv_order) {
   extern __shared__ float smem[];
   float* qs = smem;                    // [hd]
-  float* probs = qs + hd;              // [AG_THREADS]
-  float* partial = probs + AG_THREADS; // [AG_THREADS]
-  __shared__ float scratch[AG_THREADS / BH_WAVE];
+  float* probs = qs + hd;              // [THREADS]
+  float* partial = probs + THREADS; // [THREADS]
+  __shared__ float scratch[THREADS / BH_WAVE];
 
   const int row = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   const int kv_head = head / (H / KVH);
@@ -754,16 +754,16 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
 
   const T* qr = q + ((size_t)row * H + head) * hd;
-  for (int i = tid; i < hd; i += AG_THREADS) qs[i] = to_f32(qr[i]);
+  for (int i = tid; i < hd; i += THREADS) qs[i] = to_f32(qr[i]);
   __syncthreads();
 
   // value phase: groups of hd threads; group g takes keys g, g + n_groups, ... of a chunk
-  const int n_groups = AG_THREADS / hd > 0 ? AG_THREADS / hd : 1;
+  const int n_groups = THREADS / hd > 0 ? THREADS / hd : 1;
   const int group = tid / hd, dim = tid % hd;
-  const bool value_thread = tid < n_groups * hd;  // hd <= AG_THREADS is checked on the host
+  const bool value_thread = tid < n_groups * hd;  // hd <= THREADS is checked on the host
 
   float run_max = -INFINITY, run_sum = 0.f, acc = 0.f;
-  for (int c0 = first; c0 <= pos; c0 += AG_THREADS) {
+  for (int c0 = first; c0 <= pos; c0 += THREADS) {
     const int j = c0 + tid;
     float s = -INFINITY;
     if (j <= pos) {
@@ -783,7 +783,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     run_max = new_max;
     if (value_thread) {
       acc *= alpha;
-      const int n_keys = (pos - c0 + 1 < AG_THREADS) ? pos - c0 + 1 : AG_THREADS;
+      const int n_keys = (pos - c0 + 1 < THREADS) ? pos - c0 + 1 : THREADS;
       for (int jj = group; jj < n_keys; jj += n_groups) {
         const int key = c0 + jj;
         const int page = table[key / BH_PAGE];
@@ -809,23 +809,29 @@ extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const v
                                     hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "attention: sizes must be positive");
   BH_REQUIRE(H % KVH == 0, "attention: %d query heads do not group evenly into %d kv heads", H, KVH);
-  BH_REQUIRE(hd <= AG_THREADS, "attention: head size %d is above the limit of %d", hd, AG_THREADS);
+  BH_REQUIRE(hd <= 1024, "attention: head size %d is above the limit of 1024", hd);
   BH_REQUIRE(H <= 65535, "attention: too many heads");
   BH_REQUIRE(window >= 0, "attention: window must not be negative");
   BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
              "attention: cache order %d does not exist for head size %d", kv_order, hd);
-  dim3 grid(n_rows, H), block(AG_THREADS);
-  const size_t smem = (size_t)(hd + 2 * AG_THREADS) * sizeof(float);
-  if (dtype == BH_F32)
-    attention_generic_kernel<float><<<grid, block, smem, stream>>>(
-        (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, page_table, table_stride,
-        row_seq, positions, H, KVH, hd, scale, window, kv_order);
-  else if (dtype == BH_BF16)
-    attention_generic_kernel<bf16_t><<<grid, block, smem, stream>>>(
-        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table,
-        table_stride, row_seq, positions, H, KVH, hd, scale, window, kv_order);
-  else
-    return bh_fail("attention: unknown dtype %d", dtype);
+  const int threads = hd <= AG_THREADS ? AG_THREADS : (hd <= 512 ? 512 : 1024);
+  dim3 grid(n_rows, H), block(threads);
+  const size_t smem = (size_t)(hd + 2 * threads) * sizeof(float);
+#define BH_AG(T, THREADS)                                                                                             \
+  attention_generic_kernel<T, THREADS><<<grid, block, smem, stream>>>((const T*)q, (T*)out, (const T*)k_pages, (const T*)v_pages, \
+                                                                      page_table, table_stride, row_seq, positions, H, KVH, hd,  \
+                                                                      scale, window, kv_order)
+#define BH_AG_SIZES(T)                        \
+  do {                                        \
+    if (threads == AG_THREADS) BH_AG(T, AG_THREADS); \
+    else if (threads == 512) BH_AG(T, 512);   \
+    else BH_AG(T, 1024);                      \
+  } while (0)
+  if (dtype == BH_F32) BH_AG_SIZES(float);
+  else if (dtype == BH_BF16) BH_AG_SIZES(bf16_t);
+  else return bh_fail("attention: unknown dtype %d", dtype);
+#undef BH_AG_SIZES
+#undef BH_AG
   return bh_check_launch("attention_generic");
 }
 

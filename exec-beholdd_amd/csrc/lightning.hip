@@ -2,26 +2,40 @@
 //   S_t = decay_h * S_(t-1) + k_t v_t^T        S [dim][vdim] per (sequence, head), kept between steps
 //   o_t = S_t^T q_t
 // with q, k, v = silu of the rows of one fused projection.  The state, the decay and both products are float32
-// (plain FMA) whatever type the projection rows have.  A workgroup owns a tile of up to 64 value columns of one
+// (plain FMA) whatever type the projection rows have.  A workgroup owns a tile of VT value columns of one
 // (sequence, head) and walks that sequence's rows of the step in order; a thread owns a slice of `dim` of one
 // column, so the state lives in registers from the first row to the last and memory sees it once each way.
-// A stage of LN_TOKENS rows goes through LDS at a time (q and k are read by all lanes of a wave at the same
-// address, v by each lane at its own), the partial sums of the slices of `dim` are added up through LDS in a
-// fixed order.  Steps of one row a sequence (decoding) are the same kernel: one stage of one row.
+// The tile is as narrow as it takes to give every compute unit a workgroup (a prompt of one sequence has only
+// heads x vdim / VT of them), the slices as short as it takes to make the workgroup four waves.
+// A stage of LN_TOKENS rows goes through LDS at a time (q and k are read by all lanes of a slice at the same
+// address, v by each lane at its own) while the next stage's rows are already on their way into registers; the
+// partial sums of the slices of `dim` are added up through LDS in a fixed order.
+// Within a stage that starts from the state S, row t (0-based) has S_t = decay^(t+1) (S + sum_(j<=t) decay^-(j+1) k_j v_j^T):
+// with k'_j = decay^-(j+1) k_j and q'_t = decay^(t+1) q_t the inner loop is S' += k'_t v_t^T, o_t = S'^T q'_t, two
+// FMAs an element instead of three, and S' is scaled by decay^n once when the stage ends.  decay^-16 must stay a
+// modest number for that: heads that forget faster than 0.5 a row take the recurrence as written.
+// Steps of one row a sequence (decoding) are the same kernel: one stage of one row.
 #include "common.h"
 
 #define LN_TOKENS 16
+#define LN_SCALED_FROM 0.5f
 
-__device__ inline float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+// x / (1 + exp(-x)) with the hardware's reciprocal (one ulp) in place of a division of a dozen instructions
+__device__ inline float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.0f + expf(-x)); }
 
 // DPT: elements of `dim` a thread owns; VT: value columns a workgroup owns (lanes j = tid % VT); blockDim = VT * parts.
+// (Workgroups have at most 256 threads unless a slice of 64 is not enough for `dim`: saying so gives the state, the
+// prefetched stage and its places the registers they need; with the default bound of 1,024 threads they went to scratch.)
 template <typename T, int DPT, int VT>
-__global__ void lightning_scan_kernel(const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off,
+__global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off,
                                       float* __restrict__ state, const float* __restrict__ decay,
                                       const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
                                       float* __restrict__ out, int H, int dim, int vdim, int parts) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
+  __shared__ float grow[LN_TOKENS], shrink[LN_TOKENS];      // decay^(t+1) and its inverse
+  constexpr int PRE = (2 * LN_TOKENS * DPT + VT - 1) / VT + LN_TOKENS;      // a stage's elements a thread, at most
   const int seq = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const int threads = blockDim.x;
   const int j = threadIdx.x % VT, part = threadIdx.x / VT;
   const int column = tile * VT + j;
   const int padded = parts * DPT;                 // dim rounded up to whole slices; the padding holds zeros
@@ -32,6 +46,13 @@ __global__ void lightning_scan_kernel(const T* __restrict__ proj, int row_stride
   const int lo = seq_start[seq], hi = seq_start[seq + 1];
   const int slot = seq_slot[seq];
   const float lambda = decay[head];
+  const bool scaled = lambda >= LN_SCALED_FROM;
+  if (threadIdx.x < LN_TOKENS) {
+    float power = lambda;
+    for (int t = 0; t < (int)threadIdx.x; ++t) power *= lambda;
+    grow[threadIdx.x] = scaled ? power : 1.f;
+    shrink[threadIdx.x] = scaled ? 1.0f / power : 1.f;
+  }
   float* mine = state + (((size_t)slot * H + head) * dim) * vdim;
   const bool live = column < vdim;
   float s[DPT];
@@ -40,21 +61,82 @@ __global__ void lightning_scan_kernel(const T* __restrict__ proj, int row_stride
     const int i = part * DPT + e;
     s[e] = (live && i < dim) ? mine[(size_t)i * vdim + column] : 0.f;
   }
+  // A stage's elements in one numbering, row after row: q [padded], k [padded], v [VT] of each row.  Where a thread's
+  // elements come from (the column of a projected row, -1 for padding) and go to (the place in LDS) is worked out
+  // once: the divisions are by run-time numbers.
+  const int per_row = 2 * padded + VT, q_end = LN_TOKENS * padded, k_end = 2 * LN_TOKENS * padded;
+  int src[PRE], dst[PRE], tok[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    const int e = threadIdx.x + i * threads;
+    const int t = e / per_row, r = e % per_row;
+    tok[i] = t < LN_TOKENS ? t : LN_TOKENS;
+    if (r < padded) {
+      dst[i] = t * padded + r;
+      src[i] = r < dim ? q_off + head * dim + r : -1;
+    } else if (r < 2 * padded) {
+      dst[i] = q_end + t * padded + (r - padded);
+      src[i] = r - padded < dim ? k_off + head * dim + (r - padded) : -1;
+    } else {
+      dst[i] = k_end + t * VT + (r - 2 * padded);
+      src[i] = tile * VT + (r - 2 * padded) < vdim ? v_off + head * vdim + tile * VT + (r - 2 * padded) : -1;
+    }
+  }
+  // (`src` becomes the element's offset from the stage's first row.)  Every load is issued whether its element exists or
+  // not, from a place that does, and masked afterwards: loads under a branch each waited for the one before.
+  const int pre = (LN_TOKENS * per_row + threads - 1) / threads;      // elements a thread really has (<= PRE)
+  __syncthreads();      // the powers are written
+  float mul[PRE];       // what an element is multiplied by on its way into LDS: decay^(t+1) for q, its inverse for k
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    src[i] = src[i] >= 0 ? tok[i] * row_stride + src[i] : -1;
+    const int t = tok[i] < LN_TOKENS ? tok[i] : 0;
+    mul[i] = dst[i] < q_end ? grow[t] : (dst[i] < k_end ? shrink[t] : 1.f);
+  }
+  float raw[PRE];
+  auto fetch = [&](int r0) {
+    const int n = hi - r0 < LN_TOKENS ? hi - r0 : LN_TOKENS;
+    const T* first = proj + (size_t)r0 * row_stride;
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      const bool there = tok[i] < n && src[i] >= 0;
+      const float value = to_f32(first[there ? src[i] : 0]);
+      raw[i] = there ? value : 0.f;
+    }
+  };
+  auto stage = [&](int n) {
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      if (i < pre && tok[i] < n) lds[dst[i]] = silu_f32(raw[i]) * mul[i];
+    }
+  };
+  if (lo < hi) fetch(lo);
   for (int r0 = lo; r0 < hi; r0 += LN_TOKENS) {
     const int n = hi - r0 < LN_TOKENS ? hi - r0 : LN_TOKENS;
-    __syncthreads();      // the stage before has been read
-    for (int e = threadIdx.x; e < n * padded; e += blockDim.x) {
-      const int t = e / padded, i = e % padded;
-      const T* row = proj + (size_t)(r0 + t) * row_stride + (size_t)head * dim + i;
-      qs[e] = i < dim ? silu_f32(to_f32(row[q_off])) : 0.f;
-      ks[e] = i < dim ? silu_f32(to_f32(row[k_off])) : 0.f;
-    }
-    for (int e = threadIdx.x; e < n * VT; e += blockDim.x) {
-      const int t = e / VT, c = tile * VT + e % VT;
-      vs[e] = c < vdim ? silu_f32(to_f32(proj[(size_t)(r0 + t) * row_stride + v_off + (size_t)head * vdim + c])) : 0.f;
-    }
+    __syncthreads();      // the stage before has been read (and the powers are written)
+    stage(n);
     __syncthreads();
-    for (int t = 0; t < n; ++t) {
+    if (r0 + LN_TOKENS < hi) fetch(r0 + LN_TOKENS);      // on its way while this stage is computed
+    auto row_scaled = [&](int t) {
+      const float v = vs[t * VT + j];
+      const float* kt = ks + t * padded + part * DPT;
+      const float* qt = qs + t * padded + part * DPT;
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < DPT; e += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(kt + e), q4 = *reinterpret_cast<const float4*>(qt + e);
+        s[e] = fmaf(k4.x, v, s[e]);
+        s[e + 1] = fmaf(k4.y, v, s[e + 1]);
+        s[e + 2] = fmaf(k4.z, v, s[e + 2]);
+        s[e + 3] = fmaf(k4.w, v, s[e + 3]);
+        acc = fmaf(s[e], q4.x, acc);
+        acc = fmaf(s[e + 1], q4.y, acc);
+        acc = fmaf(s[e + 2], q4.z, acc);
+        acc = fmaf(s[e + 3], q4.w, acc);
+      }
+      sums[(t * parts + part) * VT + j] = acc;
+    };
+    auto row_plain = [&](int t) {
       const float v = vs[t * VT + j];
       const float* kt = ks + t * padded + part * DPT;
       const float* qt = qs + t * padded + part * DPT;
@@ -65,9 +147,22 @@ __global__ void lightning_scan_kernel(const T* __restrict__ proj, int row_stride
         acc = fmaf(s[e], qt[e], acc);
       }
       sums[(t * parts + part) * VT + j] = acc;
+    };
+    if (scaled) {
+      if (n == LN_TOKENS) {      // a whole stage: a trip count the compiler knows, so that it reads rows ahead
+#pragma unroll 4
+        for (int t = 0; t < LN_TOKENS; ++t) row_scaled(t);
+      } else {
+        for (int t = 0; t < n; ++t) row_scaled(t);
+      }
+      const float back = grow[n - 1];
+#pragma unroll
+      for (int e = 0; e < DPT; ++e) s[e] *= back;
+    } else {
+      for (int t = 0; t < n; ++t) row_plain(t);
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < n * VT; e += blockDim.x) {
+    for (int e = threadIdx.x; e < n * VT; e += threads) {
       const int t = e / VT, c = tile * VT + e % VT;
       if (c >= vdim) continue;
       float total = 0.f;
@@ -84,47 +179,112 @@ __global__ void lightning_scan_kernel(const T* __restrict__ proj, int row_stride
   }
 }
 
-template <typename T, int DPT>
+// A step of one row a sequence (decoding): the same tiles and slices, but nothing to prefetch and no stage to walk, so
+// none of the registers that hold a stage's places: the state streams through at several workgroups a compute unit.
+template <typename T, int DPT, int VT>
+__global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_step_kernel(
+    const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off, float* __restrict__ state,
+    const float* __restrict__ decay, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
+    float* __restrict__ out, int H, int dim, int vdim, int parts) {
+  extern __shared__ __align__(16) float lds[];
+  const int seq = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const int j = threadIdx.x % VT, part = threadIdx.x / VT;
+  const int column = tile * VT + j, padded = parts * DPT;
+  float* qs = lds;              // [padded]
+  float* ks = qs + padded;      // [padded]
+  float* vs = ks + padded;      // [VT]
+  float* sums = vs + VT;        // [parts][VT]
+  const int row = seq_start[seq];
+  if (seq_start[seq + 1] <= row) return;
+  const float lambda = decay[head];
+  float* mine = state + (((size_t)seq_slot[seq] * H + head) * dim) * vdim;
+  const bool live = column < vdim;
+  float s[DPT];
+#pragma unroll
+  for (int e = 0; e < DPT; ++e) {
+    const int i = part * DPT + e;
+    s[e] = (live && i < dim) ? mine[(size_t)i * vdim + column] : 0.f;
+  }
+  const T* from = proj + (size_t)row * row_stride;
+  for (int i = threadIdx.x; i < padded; i += blockDim.x) {
+    qs[i] = i < dim ? silu_f32(to_f32(from[q_off + head * dim + i])) : 0.f;
+    ks[i] = i < dim ? silu_f32(to_f32(from[k_off + head * dim + i])) : 0.f;
+  }
+  for (int c = threadIdx.x; c < VT; c += blockDim.x)
+    vs[c] = tile * VT + c < vdim ? silu_f32(to_f32(from[v_off + head * vdim + tile * VT + c])) : 0.f;
+  __syncthreads();
+  const float v = vs[j];
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < DPT; ++e) {
+    s[e] = fmaf(lambda, s[e], ks[part * DPT + e] * v);
+    acc = fmaf(s[e], qs[part * DPT + e], acc);
+  }
+  sums[part * VT + j] = acc;
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < DPT; ++e) {
+      const int i = part * DPT + e;
+      if (i < dim) mine[(size_t)i * vdim + column] = s[e];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < VT && tile * VT + threadIdx.x < vdim) {
+    float total = 0.f;
+    for (int p = 0; p < parts; ++p) total += sums[p * VT + threadIdx.x];
+    out[((size_t)row * H + head) * vdim + tile * VT + threadIdx.x] = total;
+  }
+}
+
+template <typename T, int DPT, int VT>
 static int launch_lightning(const void* proj, int row_stride, int q_off, int k_off, int v_off, float* state,
                             const float* decay, const int32_t* seq_start, const int32_t* seq_slot, float* out, int n_seqs,
-                            int H, int dim, int vdim, hipStream_t stream) {
+                            int n_rows, int H, int dim, int vdim, hipStream_t stream) {
   const int parts = (dim + DPT - 1) / DPT;
-  const int vt = vdim > 32 ? 64 : (vdim > 16 ? 32 : 16);
-  BH_REQUIRE(parts * vt <= 1024, "lightning: heads of %d x %d need more than 1024 threads", dim, vdim);
-  const int tiles = (vdim + vt - 1) / vt;
-  const size_t smem = (size_t)LN_TOKENS * (2 * parts * DPT + vt + parts * vt) * sizeof(float);
-  BH_REQUIRE(smem <= 64 * 1024, "lightning: heads of %d x %d need %zu bytes of LDS", dim, vdim, smem);
-  dim3 grid(n_seqs, H, tiles), block(parts * vt);
-#define BH_SCAN(VT)                                                                                               \
-  lightning_scan_kernel<T, DPT, VT><<<grid, block, smem, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, \
-                                                                   state, decay, seq_start, seq_slot, out, H, dim, vdim, parts)
-  if (vt == 64) BH_SCAN(64);
-  else if (vt == 32) BH_SCAN(32);
-  else BH_SCAN(16);
-#undef BH_SCAN
+  BH_REQUIRE(parts * VT <= 1024, "lightning: heads of %d x %d need more than 1024 threads", dim, vdim);
+  const int tiles = (vdim + VT - 1) / VT;
+  const size_t smem = (size_t)LN_TOKENS * (2 * parts * DPT + VT + parts * VT) * sizeof(float);
+  BH_REQUIRE(smem <= 63 * 1024, "lightning: heads of %d x %d need %zu bytes of LDS", dim, vdim, smem);
+  dim3 grid(n_seqs, H, tiles), block(parts * VT);
+  if (n_rows == n_seqs) {      // one row each
+    const size_t lean = (size_t)(2 * parts * DPT + VT + parts * VT) * sizeof(float);
+    lightning_step_kernel<T, DPT, VT><<<grid, block, lean, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, state, decay,
+                                                                     seq_start, seq_slot, out, H, dim, vdim, parts);
+    return bh_check_launch("lightning_step");
+  }
+  lightning_scan_kernel<T, DPT, VT><<<grid, block, smem, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, state, decay,
+                                                                   seq_start, seq_slot, out, H, dim, vdim, parts);
   return bh_check_launch("lightning_scan");
 }
 
 // proj [n_rows][row_stride]: a row holds q (H x dim) from q_off, k (H x dim) from k_off, v (H x vdim) from v_off, all
 // before their silu.  state [slots][H][dim][vdim] float32; rows seq_start[b] .. seq_start[b + 1] - 1 belong to the
-// sequence in slot seq_slot[b], in order.  out [n_rows][H * vdim] float32.
+// sequence in slot seq_slot[b], in order, and every sequence has at least one.  out [n_rows][H * vdim] float32.
 extern "C" int bh_lightning_scan(const void* proj, int dtype, int row_stride, int q_off, int k_off, int v_off, float* state,
                                  const float* decay, const int32_t* seq_start, const int32_t* seq_slot, float* out,
-                                 int n_seqs, int H, int dim, int vdim, hipStream_t stream) {
-  BH_REQUIRE(n_seqs > 0 && H > 0 && dim > 0 && vdim > 0, "lightning: sizes must be positive");
+                                 int n_seqs, int n_rows, int H, int dim, int vdim, hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && n_rows >= n_seqs && H > 0 && dim > 0 && vdim > 0,
+             "lightning: sizes must be positive, and every sequence of the step brings a row");
   BH_REQUIRE(H <= 65535 && n_seqs <= 2147483647, "lightning: too many heads");
   BH_REQUIRE(dim <= 1024, "lightning: a key size of %d is above the limit of 1024", dim);
   BH_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + H * dim <= row_stride && k_off + H * dim <= row_stride &&
                  v_off + H * vdim <= row_stride,
              "lightning: q, k and v do not lie inside a row of %d", row_stride);
-  const int quarter = (dim + 3) / 4;     // four slices of dim a column where that keeps a slice short
-#define BH_LN(T, DPT) \
-  return launch_lightning<T, DPT>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, H, dim, vdim, stream)
-#define BH_LN_SIZES(T)              \
-  if (quarter <= 4) BH_LN(T, 4);    \
-  if (quarter <= 8) BH_LN(T, 8);    \
-  if (quarter <= 16) BH_LN(T, 16);  \
-  if (quarter <= 32) BH_LN(T, 32);  \
+  // value columns a workgroup: 64 where that many workgroups fill the chip twice, else fewer, down to 16
+  int vt = vdim > 32 ? 64 : (vdim > 16 ? 32 : 16);
+  while (vt > 16 && (long)n_seqs * H * ((vdim + vt - 1) / vt) < 2L * bh_compute_units()) vt /= 2;
+  const int slice = (dim + 256 / vt - 1) / (256 / vt);      // slices of dim that make the workgroup four waves
+#define BH_LN(T, DPT)                                                                                                   \
+  do {                                                                                                                  \
+    if (vt == 64) return launch_lightning<T, DPT, 64>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
+    if (vt == 32) return launch_lightning<T, DPT, 32>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
+    return launch_lightning<T, DPT, 16>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
+  } while (0)
+#define BH_LN_SIZES(T)            \
+  if (slice <= 4) BH_LN(T, 4);    \
+  if (slice <= 8) BH_LN(T, 8);    \
+  if (slice <= 16) BH_LN(T, 16);  \
+  if (slice <= 32) BH_LN(T, 32);  \
   BH_LN(T, 64)
   if (dtype == BH_F32) { BH_LN_SIZES(float); }
   if (dtype == BH_BF16) { BH_LN_SIZES(bf16_t); }

@@ -166,7 +166,7 @@ class KernelSizes:
             "bh_streams_update": [p, p, p, p, p, i, i, i, p],
             "bh_scale": [p, ctypes.c_long, f, p],
             "bh_relu_squared": [p, i, ctypes.c_long, p],
-            "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, p],
+            "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, i, p],
             "bh_gated_rmsnorm": [p, p, i, i, p, p, i, i, f, i, p],
             "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, p],
             "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, p],
@@ -813,7 +813,7 @@ class HipKernels(KernelSizes):
             self._ptr(proj, "lightning proj"), _code(proj, "lightning proj"), stride, int(q_off), int(k_off), int(v_off),
             self._ptr(state, "lightning state", f32), self._ptr(decay, "lightning decay", f32),
             self._ptr(seq_start, "seq_start", i32), self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "lightning out", f32),
-            n_seqs, n_heads, dim, vdim, self._stream()))
+            n_seqs, n_rows, n_heads, dim, vdim, self._stream()))
 
     def gated_rmsnorm(self, o, proj, gate_off, weight, eps, out):
         """out[r] = RMSNorm(o[r]) * weight * sigmoid(proj[r, gate_off : gate_off + W]); o f32 [n, W], out [n, W] in the

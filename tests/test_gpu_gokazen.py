@@ -202,6 +202,8 @@ ALONE = {
                "layers": [gm.latent(5, 24, 8, 40, 56, 0.8, base=300.0)]},
     "latent, half turned": {"architecture": "Gokazen", "vocab": 61, "width": 40, "logit_scale": 1.0, "norm": {"eps": 1e-5},
                             "layers": [gm.latent(2, 8, 24, 16, 72, 1.1, base=1e5, dims=12)]},
+    "latent, wide": {"architecture": "Gokazen", "vocab": 61, "width": 40, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+                     "layers": [gm.latent(2, 8, 8, 16, 280, 0.5)]},        # a cached head of 288: beyond the matrix-core attention's sizes
     "feed-forward": {"architecture": "Gokazen", "vocab": 61, "width": 40, "streams": 2, "logit_scale": 2.0, "norm": {"eps": 1e-5},
                      "layers": [gm.lightning(1, 4, 4, [0.5], ff=100)]},
 }
