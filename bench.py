@@ -314,16 +314,15 @@ def gokazen_kernels(K, torch, width, heads, rank, rot, context, streams=2):
         qd = torch.randn(rows, heads * q_head + kv_head, device=dev).to(bf16)
         k_pages, v_pages, table = pages_for(seqs, past + each, 1, kv_head)
         freq, latent_weight = torch.ones(rot // 2, device=dev), torch.ones(rank, device=dev)
-        us = timed(lambda: K.latent_write(qd, heads * q_head, latent_weight, 1e-6, freq, rot, positions, row_seq,
-                                          k_pages, v_pages, table, rank, rot), torch)
-        note(f"latent_write, {tag}", us, rows * kv_head * 2 * 3)
-        key_up = torch.randn(heads, dim, rank, device=dev).to(bf16)
         query = torch.empty(rows, heads * kv_head, device=dev, dtype=bf16)
+        us = timed(lambda: K.latent_write(qd, heads * q_head, latent_weight, 1e-6, freq, rot, positions, row_seq, k_pages, v_pages,
+                                          table, rank, rot, query=query, query_head=kv_head, query_first=rank, source_head=q_head,
+                                          source_first=dim, n_heads=heads), torch)
+        note(f"latent_write with the queries' rotation, {tag}", us, rows * kv_head * 2 * 3 + 2 * rows * heads * rot * 2)
+        key_up = torch.randn(heads, dim, rank, device=dev).to(bf16)
         us = timed(lambda: K.heads_linear(qd, q_head, 0, key_up, query, kv_head, 0, heads), torch)
         note(f"heads_linear (queries into the latent), {tag}", us, key_up.numel() * 2 + rows * heads * (dim + rank) * 2,
              2.0 * rows * heads * dim * rank, PEAK_FLOPS["bf16"])
-        us = timed(lambda: K.rotate_heads(qd, q_head, dim, query, kv_head, rank, freq, rot, positions, heads, rot), torch)
-        note(f"rotate_heads, {tag}", us, 2 * rows * heads * rot * 2)
         attended = torch.empty_like(query)
         scale = (dim + rot) ** -0.5
         us = timed(lambda: K.attention(query, attended, k_pages, v_pages, table, row_seq, positions, heads, 1, kv_head, scale, 0, layout=layout), torch)
@@ -336,7 +335,8 @@ def gokazen_kernels(K, torch, width, heads, rank, rot, context, streams=2):
         note(f"heads_linear (latents into values), {tag}", us, value_up.numel() * 2 + rows * heads * (rank + vdim) * 2,
              2.0 * rows * heads * rank * vdim, PEAK_FLOPS["bf16"])
         inner = torch.randn(rows, 3 * width, device=dev).to(bf16)
-        us = timed(lambda: K.relu_squared(inner), torch)
+        activated_sq = torch.empty_like(inner)
+        us = timed(lambda: K.relu_squared(inner, activated_sq), torch)
         note(f"relu_squared, {tag}", us, 2 * inner.numel() * 2)
         # -- their like in Qwen3 at the same width: 4 query heads of 128 to a kv head
         kv_heads = max(heads // 4, 1)

@@ -16,11 +16,31 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     const T* __restrict__ down, int row_stride, int offset, const float* __restrict__ w, float eps,
     const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     T* __restrict__ k_pages, T* __restrict__ v_pages, const int32_t* __restrict__ page_table, int table_stride, int rank,
-    int rot_dim, int kv_order) {
+    int rot_dim, int kv_order, int write, T* __restrict__ query, long q_row, int q_head, int q_first, int src_head, int src_first,
+    int H) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const T* x = down + (size_t)row * row_stride + offset;
   const int pos = positions[row], hd = rank + rot_dim;
+  const int half = turned / 2;
+  if (query != nullptr) {      // the heads' rotated query parts, from the same projected row
+    for (int e = threadIdx.x; e < H * rot_dim; e += blockDim.x) {
+      const int head = e / rot_dim, i = e % rot_dim;
+      const T* from = down + (size_t)row * row_stride + (size_t)head * src_head + src_first;
+      float y;
+      if (i < turned) {
+        const int pair = i < half ? i : i - half;
+        const float angle = (float)pos * freq[pair];
+        const float c = cosf(angle), s = sinf(angle);
+        const float u = to_f32(from[pair]), v = to_f32(from[pair + half]);
+        y = i < half ? u * c - v * s : v * c + u * s;
+      } else {
+        y = to_f32(from[i]);
+      }
+      query[(size_t)row * q_row + (size_t)head * q_head + q_first + i] = from_f32<T>(y);
+    }
+  }
+  if (!write) return;
   const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE], token = pos % BH_PAGE;
   T* keys = k_pages + (size_t)page * BH_PAGE * hd;
   T* values = v_pages + (size_t)page * BH_PAGE * hd;
@@ -36,7 +56,6 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     keys[bh_key_index(kv_order, token, i, hd)] = c;
     values[bh_value_index(kv_order, token, i, hd)] = c;
   }
-  const int half = turned / 2;
   for (int i = threadIdx.x; i < rot_dim; i += blockDim.x) {
     float y;
     if (i < turned) {
@@ -54,11 +73,18 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
 }
 
 // down [n_rows][row_stride]: a row holds, from `offset`, rank latent elements and rot_dim key elements.
-// Pages as the attention kernels take them for one kv head of size rank + rot_dim.
+// Pages as the attention kernels take them for one kv head of size rank + rot_dim (written when `write` is set).
+// With `query`, the same launch rotates the rot_dim elements at src_first of each of the H heads (src_head apart) of the
+// same row into query[row][head * q_head + q_first ..]: the heads' rotated query parts, beside the key's.
 extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int offset, const float* w, float eps,
                                const float* freq, int turned, const int32_t* positions, const int32_t* row_seq,
                                void* k_pages, void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
-                               int rank, int rot_dim, int kv_order, hipStream_t stream) {
+                               int rank, int rot_dim, int kv_order, int write, void* query, long q_row, int q_head, int q_first,
+                               int src_head, int src_first, int H, hipStream_t stream) {
+  BH_REQUIRE(write || query != nullptr, "latent_write: nothing to do");
+  BH_REQUIRE(query == nullptr || (H > 0 && q_first >= 0 && src_first >= 0 && q_first + rot_dim <= q_head && src_first + rot_dim <= src_head &&
+                                  (long)H * q_head <= q_row && H * src_head <= row_stride),
+             "latent_write: the heads' rotated slices do not lie inside their rows");
   BH_REQUIRE(n_rows > 0 && rank > 0 && rot_dim > 0, "latent_write: sizes must be positive");
   BH_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= rot_dim, "latent_write: %d turned dimensions of %d", turned, rot_dim);
   BH_REQUIRE(turned == 0 || freq != nullptr, "latent_write: a rotation needs its frequencies");
@@ -68,7 +94,8 @@ extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int 
 #define BH_LW(T)                                                                                                      \
   latent_write_kernel<T><<<dim3(n_rows), dim3(256), 0, stream>>>((const T*)down, row_stride, offset, w, eps, freq, turned, \
                                                                  positions, row_seq, (T*)k_pages, (T*)v_pages, page_table, \
-                                                                 table_stride, rank, rot_dim, kv_order)
+                                                                 table_stride, rank, rot_dim, kv_order, write, (T*)query, q_row, q_head, \
+                                                                 q_first, src_head, src_first, H)
   if (dtype == BH_F32) BH_LW(float);
   else if (dtype == BH_BF16) BH_LW(bf16_t);
   else return bh_fail("latent_write: unknown dtype %d", dtype);
@@ -80,13 +107,14 @@ extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int 
 // y[row][h][o] = sum_i w[h][i][o] * x[row][h][i] for o < n_out, i < n_in; x and y are slices of the heads of wider rows
 // (row stride, head stride and first element given for each); w [H][n_in][n_out], the output index running fastest,
 // so that the lanes of a wave read neighbouring weights.  Float32 sums; a workgroup takes HL_ROWS rows of one head
-// and up to 256 outputs, the rows' inputs going through LDS once.
+// and up to 256 outputs, the rows' inputs going through LDS once.  y's rows lie one after the other, or, for the
+// product that reads them next, in blocks of rows (bh_rows_index; y_row is then the matrix's width).
 #define HL_ROWS 16
 
 template <typename T>
 __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__ x, long x_row, int x_head, int x_first,
                                                            const T* __restrict__ w, T* __restrict__ y, long y_row, int y_head,
-                                                           int y_first, int n_rows, int n_in, int n_out) {
+                                                           int y_first, int n_rows, int n_in, int n_out, int y_block_rows) {
   extern __shared__ float xs[];      // [HL_ROWS][n_in]
   const int row0 = blockIdx.x * HL_ROWS, head = blockIdx.y, o = blockIdx.z * 256 + threadIdx.x;
   const int rows = n_rows - row0 < HL_ROWS ? n_rows - row0 : HL_ROWS;
@@ -105,11 +133,15 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__
   }
 #pragma unroll
   for (int r = 0; r < HL_ROWS; ++r)
-    if (r < rows) y[(size_t)(row0 + r) * y_row + (size_t)head * y_head + y_first + o] = from_f32<T>(acc[r]);
+    if (r < rows) y[bh_rows_index(y_block_rows, row0 + r, head * y_head + y_first + o, (int)y_row)] = from_f32<T>(acc[r]);
 }
 
 extern "C" int bh_heads_linear(const void* x, long x_row, int x_head, int x_first, const void* w, void* y, long y_row,
-                               int y_head, int y_first, int dtype, int n_rows, int H, int n_in, int n_out, hipStream_t stream) {
+                               int y_head, int y_first, int dtype, int n_rows, int H, int n_in, int n_out, int y_block_rows,
+                               hipStream_t stream) {
+  BH_REQUIRE(y_block_rows == 0 || ((y_block_rows == 8 || y_block_rows == 16) && dtype == BH_BF16 && y_row % 32 == 0 && y_row < (1L << 31)),
+             "heads_linear: an output in blocks of %d rows needs bfloat16 and rows of a multiple of 32 elements (got %ld)",
+             y_block_rows, y_row);
   BH_REQUIRE(n_rows > 0 && H > 0 && n_in > 0 && n_out > 0, "heads_linear: sizes must be positive");
   BH_REQUIRE(H <= 65535 && (n_out + 255) / 256 <= 65535, "heads_linear: too many heads or outputs");
   BH_REQUIRE(x_first >= 0 && y_first >= 0 && x_first + n_in <= x_head && y_first + n_out <= y_head &&
@@ -120,7 +152,7 @@ extern "C" int bh_heads_linear(const void* x, long x_row, int x_head, int x_firs
   dim3 grid((n_rows + HL_ROWS - 1) / HL_ROWS, H, (n_out + 255) / 256), block(256);
 #define BH_HL(T)                                                                                                         \
   heads_linear_kernel<T><<<grid, block, smem, stream>>>((const T*)x, x_row, x_head, x_first, (const T*)w, (T*)y, y_row, y_head, \
-                                                        y_first, n_rows, n_in, n_out)
+                                                        y_first, n_rows, n_in, n_out, y_block_rows)
   if (dtype == BH_F32) BH_HL(float);
   else if (dtype == BH_BF16) BH_HL(bf16_t);
   else return bh_fail("heads_linear: unknown dtype %d", dtype);

@@ -139,6 +139,101 @@ extern "C" int bh_streams_update(float* x, const float* y, const float* mix, con
   return bh_check_launch("streams_update");
 }
 
+// ---- write, and read for the sublayer that follows, in one pass ---------------------------------------------------
+// streams_update for one row, then streams_rmsnorm of the row as it has become (with the next sublayer's `take` and
+// norm weight): a workgroup per row; a thread keeps the next sublayer's sum of its elements while it writes the streams.
+template <typename TO, int PER>
+__global__ void streams_update_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ mix,
+                                              const float* __restrict__ give, const float* __restrict__ scale,
+                                              const float* __restrict__ take, const float* __restrict__ w, TO* __restrict__ out,
+                                              int width, int streams, float eps, int block_rows) {
+  __shared__ float scratch[16];
+  __shared__ float m[BH_STREAMS_MOST * BH_STREAMS_MOST];
+  __shared__ float g[BH_STREAMS_MOST], share[BH_STREAMS_MOST];
+  const int r = blockIdx.x;
+  for (int e = threadIdx.x; e < streams * streams; e += blockDim.x) m[e] = mix ? mix[e] : (e / streams == e % streams ? 1.f : 0.f);
+  if (threadIdx.x < streams) {
+    g[threadIdx.x] = give ? give[threadIdx.x] : 1.f;
+    share[threadIdx.x] = take ? take[threadIdx.x] : 1.f;
+  }
+  __syncthreads();
+  float* xr = x + (size_t)r * streams * width;
+  const float* yr = y + (size_t)r * width;
+  auto renew = [&](int i) {      // the streams' element i as it becomes, written; returns the next sublayer's sum of it
+    float old[BH_STREAMS_MOST];
+    for (int s = 0; s < streams; ++s) old[s] = xr[(size_t)s * width + i];
+    const float add = (scale ? scale[i] : 1.f) * yr[i];
+    float u = 0.f;
+    for (int t = 0; t < streams; ++t) {
+      float v = 0.f;
+      for (int s = 0; s < streams; ++s) v = fmaf(m[s * streams + t], old[s], v);
+      v = fmaf(g[t], add, v);
+      xr[(size_t)t * width + i] = v;
+      u = fmaf(share[t], v, u);
+    }
+    return u;
+  };
+  auto at = [&](int i) { return out + bh_rows_index(block_rows, r, i, width); };
+  float ss = 0.f;
+  if (PER > 0) {
+    float uv[PER > 0 ? PER : 1];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      uv[j] = i < width ? renew(i) : 0.f;
+      ss += uv[j] * uv[j];
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      if (i < width) *at(i) = from_f32<TO>(uv[j] * inv * (w ? w[i] : 1.f));
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float u = renew(i);
+    ss += u * u;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {      // a thread reads back what it wrote itself
+    float u = 0.f;
+    for (int t = 0; t < streams; ++t) u = fmaf(share[t], xr[(size_t)t * width + i], u);
+    *at(i) = from_f32<TO>(u * inv * (w ? w[i] : 1.f));
+  }
+}
+
+extern "C" int bh_streams_update_rmsnorm(float* x, const float* y, const float* mix, const float* give, const float* scale,
+                                         const float* take, const float* w, void* out, int out_dtype, int n_rows, int width,
+                                         int streams, float eps, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "streams_update_rmsnorm: rows %d and width %d must be positive", n_rows, width);
+  BH_REQUIRE(streams >= 1 && streams <= BH_STREAMS_MOST, "streams_update_rmsnorm: 1 to %d streams, not %d", BH_STREAMS_MOST, streams);
+  BH_REQUIRE(eps >= 0.f, "streams_update_rmsnorm: eps must not be negative");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && out_dtype == BH_BF16 && width % 32 == 0),
+             "streams_update_rmsnorm: rows in blocks of %d need bfloat16 and a width that is a multiple of 32 (got %d)",
+             out_block_rows, width);
+  const int threads = width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256);
+  const int per = (width + threads - 1) / threads;
+  dim3 grid(n_rows), block(threads);
+#define BH_SUN(TO, PER)                                                                                                  \
+  streams_update_rmsnorm_kernel<TO, PER><<<grid, block, 0, stream>>>(x, y, mix, give, scale, take, w, (TO*)out, width, streams, \
+                                                                     eps, out_block_rows)
+#define BH_SUN_SIZES(TO)           \
+  do {                             \
+    if (per <= 4) BH_SUN(TO, 4);   \
+    else if (per <= 8) BH_SUN(TO, 8); \
+    else BH_SUN(TO, 0);            \
+  } while (0)
+  if (out_dtype == BH_F32) BH_SUN_SIZES(float);
+  else if (out_dtype == BH_BF16) BH_SUN_SIZES(bf16_t);
+  else return bh_fail("streams_update_rmsnorm: unknown output dtype %d", out_dtype);
+#undef BH_SUN_SIZES
+#undef BH_SUN
+  return bh_check_launch("streams_update_rmsnorm");
+}
+
 // ---- small elementwise steps ---------------------------------------------------------------------------------
 __global__ void scale_kernel(float* __restrict__ x, float factor, size_t total) {
   const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -153,21 +248,29 @@ extern "C" int bh_scale(float* x, long total, float factor, hipStream_t stream) 
   return bh_check_launch("scale");
 }
 
-// x <- max(x, 0)^2, in place, in float32 whatever the element type
+// out <- max(x, 0)^2 (out may be x itself), in float32 whatever the element type; the output's rows one after the other
+// or in blocks of rows (bh_rows_index)
 template <typename T>
-__global__ void relu_squared_kernel(T* __restrict__ x, size_t total) {
+__global__ void relu_squared_kernel(const T* __restrict__ x, T* __restrict__ out, int width, size_t total, int block_rows) {
   const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (at >= total) return;
   const float v = fmaxf(to_f32(x[at]), 0.f);
-  x[at] = from_f32<T>(v * v);
+  const size_t to = block_rows ? (size_t)bh_rows_index(block_rows, (int)(at / width), (int)(at % width), width) : at;
+  out[to] = from_f32<T>(v * v);
 }
 
-extern "C" int bh_relu_squared(void* x, int dtype, long total, hipStream_t stream) {
-  BH_REQUIRE(total > 0, "relu_squared: nothing to do");
-  const size_t blocks = ((size_t)total + 255) / 256;
+extern "C" int bh_relu_squared(const void* x, void* out, int dtype, int n_rows, int width, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "relu_squared: nothing to do");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && dtype == BH_BF16 && width % 32 == 0 && x != out),
+             "relu_squared: rows in blocks of %d need bfloat16, a width that is a multiple of 32 (got %d) and an output of their own",
+             out_block_rows, width);
+  const size_t total = (size_t)n_rows * width;
+  const size_t blocks = (total + 255) / 256;
   BH_REQUIRE(blocks <= 2147483647u, "relu_squared: too many elements");
-  if (dtype == BH_F32) relu_squared_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((float*)x, (size_t)total);
-  else if (dtype == BH_BF16) relu_squared_kernel<bf16_t><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((bf16_t*)x, (size_t)total);
+  if (dtype == BH_F32)
+    relu_squared_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((const float*)x, (float*)out, width, total, out_block_rows);
+  else if (dtype == BH_BF16)
+    relu_squared_kernel<bf16_t><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((const bf16_t*)x, (bf16_t*)out, width, total, out_block_rows);
   else return bh_fail("relu_squared: unknown dtype %d", dtype);
   return bh_check_launch("relu_squared");
 }

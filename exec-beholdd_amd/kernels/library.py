@@ -164,12 +164,13 @@ class KernelSizes:
             "bh_streams_open": [p, p, i, i, i, p],
             "bh_streams_rmsnorm": [p, p, p, p, p, i, i, i, i, f, i, p],
             "bh_streams_update": [p, p, p, p, p, i, i, i, p],
+            "bh_streams_update_rmsnorm": [p, p, p, p, p, p, p, p, i, i, i, i, f, i, p],
             "bh_scale": [p, ctypes.c_long, f, p],
-            "bh_relu_squared": [p, i, ctypes.c_long, p],
+            "bh_relu_squared": [p, p, i, i, i, i, p],
             "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, i, p],
             "bh_gated_rmsnorm": [p, p, i, i, p, p, i, i, f, i, p],
-            "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, p],
-            "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, p],
+            "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, i, i, i, i, i, p],
+            "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, i, p],
             "bh_rotate_heads": [p, ctypes.c_long, i, i, p, ctypes.c_long, i, i, i, p, i, p, i, i, i, p],
         }
         for name, argtypes in table.items():
@@ -789,13 +790,33 @@ class HipKernels(KernelSizes):
             self._ptr(mix, "streams_update mix", f32, True), self._ptr(give, "streams_update give", f32, True),
             self._ptr(scale, "streams_update scale", f32, True), n_rows, width, streams, self._stream()))
 
+    def streams_update_rmsnorm(self, x, y, mix, give, scale, take, weight, eps, out):
+        """`streams_update(x, y, mix, give, scale)` and then `streams_rmsnorm(x, take, weight, eps, out)` of every row, in one
+        pass over the streams."""
+        n_rows, streams, width = x.shape
+        if tuple(y.shape) != (n_rows, width) or tuple(out.shape) != (n_rows, width) \
+                or (mix is not None and tuple(mix.shape) != (streams, streams)) \
+                or any(t is not None and tuple(t.shape) != (streams,) for t in (give, take)) \
+                or any(t is not None and tuple(t.shape) != (width,) for t in (scale, weight)):
+            raise KernelError(f"streams_update_rmsnorm: shapes x {tuple(x.shape)}, y {tuple(y.shape)}, out {tuple(out.shape)} do not fit")
+        f32 = (torch.float32,)
+        self._check(self.lib.bh_streams_update_rmsnorm(
+            self._ptr(x, "streams x", f32), self._ptr(y, "streams y", f32), self._ptr(mix, "streams mix", f32, True),
+            self._ptr(give, "streams give", f32, True), self._ptr(scale, "streams scale", f32, True),
+            self._ptr(take, "streams take", f32, True), self._ptr(weight, "norm weight", f32, True), self._ptr(out, "norm out"),
+            _code(out, "norm out"), n_rows, width, streams, float(eps), _block_rows(out), self._stream()))
+
     def scale(self, x, factor):
         """x *= factor, in place; x float32."""
         self._check(self.lib.bh_scale(self._ptr(x, "scale x", (torch.float32,)), x.numel(), float(factor), self._stream()))
 
-    def relu_squared(self, x):
-        """x <- max(x, 0)^2, in place."""
-        self._check(self.lib.bh_relu_squared(self._ptr(x, "relu_squared x"), _code(x, "relu_squared x"), x.numel(), self._stream()))
+    def relu_squared(self, x, out=None):
+        """out <- max(x, 0)^2; in place without `out`, which may be `BlockedRows` for the product that reads it next."""
+        out = x if out is None else out
+        if x.dim() != 2 or tuple(out.shape) != tuple(x.shape) or out.dtype != x.dtype:
+            raise KernelError(f"relu_squared: shapes {tuple(x.shape)} -> {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_relu_squared(self._ptr(x, "relu_squared x"), self._ptr(out, "relu_squared out"),
+                                             _code(x, "relu_squared x"), x.shape[0], x.shape[1], _block_rows(out), self._stream()))
 
     # ---- linear attention with a decay, as a recurrence over a float32 state ----
     def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
@@ -830,15 +851,19 @@ class HipKernels(KernelSizes):
 
     # ---- attention over a cached latent ----
     def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
-                     rank, rot_dim):
+                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0):
         """From each row of `down` [n, P], at `offset`: c = RMSNorm(rank elements) * weight and the next rot_dim elements
         rotated (the first `turned` of them, pairs (i, i + turned/2), angle position * freq[i]); key [c | rotated] and
-        value [c | 0] of ONE kv head of size rank + rot_dim go into the cache pages of (sequence, position)."""
+        value [c | 0] of ONE kv head of size rank + rot_dim go into the cache pages of (sequence, position) (unless
+        `write` is False).  With `query` [n, >= n_heads * query_head] the same launch rotates the rot_dim elements at
+        `source_first` of each of the row's `n_heads` heads (`source_head` apart) into query[row, h * query_head + query_first ..]."""
         n_rows = down.shape[0]
         head = rank + rot_dim
         if positions.shape != (n_rows,) or row_seq.shape != (n_rows,) or (weight is not None and tuple(weight.shape) != (rank,)) \
                 or (freq is not None and tuple(freq.shape) != (turned // 2,)):
             raise KernelError("latent_write: one position and one sequence per row, a weight [rank] and a frequency a pair")
+        if query is not None and (query.dim() != 2 or query.shape[0] != n_rows or query.dtype != down.dtype):
+            raise KernelError(f"latent_write: the queries {tuple(query.shape)} do not fit {n_rows} rows of {down.dtype}")
         self._check_pages(k_pages, v_pages, page_table, 1, head, down.dtype, "latent_write")
         f32, i32 = (torch.float32,), (torch.int32,)
         self._check(self.lib.bh_latent_write(
@@ -846,18 +871,21 @@ class HipKernels(KernelSizes):
             self._ptr(weight, "latent norm weight", f32, True), float(eps), self._ptr(freq, "rotation frequencies", f32, True),
             int(turned), self._ptr(positions, "positions", i32), self._ptr(row_seq, "row_seq", i32),
             self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"), self._ptr(page_table, "page_table", i32),
-            page_table.shape[1], n_rows, int(rank), int(rot_dim), self.kv_order(k_pages.dtype, head), self._stream()))
+            page_table.shape[1], n_rows, int(rank), int(rot_dim), self.kv_order(k_pages.dtype, head), int(bool(write)),
+            self._ptr(query, "rotated queries", None, True), query.shape[1] if query is not None else 0, int(query_head),
+            int(query_first), int(source_head), int(source_first), int(n_heads), self._stream()))
 
     def heads_linear(self, x, x_head, x_first, w, y, y_head, y_first, n_heads):
         """y[row, h, y_first + o] = sum_i w[h, i, o] * x[row, h, x_first + i]: x [n, >= H * x_head] and y [n, >= H * y_head]
-        are rows of heads of x_head and y_head elements, w [H, n_in, n_out] of their type; float32 sums."""
+        are rows of heads of x_head and y_head elements, w [H, n_in, n_out] of their type; float32 sums.  `y` may be
+        `BlockedRows` (for the product that reads it next)."""
         n_rows = x.shape[0]
         if w.dim() != 3 or w.shape[0] != n_heads or y.shape[0] != n_rows or x.dtype != w.dtype or y.dtype != w.dtype:
             raise KernelError(f"heads_linear: shapes x {tuple(x.shape)}, w {tuple(w.shape)}, y {tuple(y.shape)} do not fit")
         self._check(self.lib.bh_heads_linear(
             self._ptr(x, "heads_linear x"), x.shape[1], int(x_head), int(x_first), self._ptr(w, "heads_linear w"),
             self._ptr(y, "heads_linear y"), y.shape[1], int(y_head), int(y_first), _code(w, "heads_linear w"), n_rows, n_heads,
-            w.shape[1], w.shape[2], self._stream()))
+            w.shape[1], w.shape[2], _block_rows(y), self._stream()))
 
     def rotate_heads(self, x, x_head, x_first, y, y_head, y_first, freq, turned, positions, n_heads, width):
         """y[row, h, y_first + i] = x[row, h, x_first + i] for i < width, the first `turned` of them rotated in pairs

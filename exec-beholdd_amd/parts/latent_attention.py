@@ -83,17 +83,17 @@ class LatentAttention:
         k = ctx.kernels
         heads, rank, turned = self.n_heads, self.kv_rank, self.rotation.dims
         proj = self.proj.forward(ctx, x)
-        if cache.writes:
-            k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, self.frequencies, turned, ctx.positions,
-                           ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table, rank, self.rot_dim)
         query = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
+        # one launch: c and k_r into the cache, and the heads' rotated query parts into their places
+        k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, self.frequencies, turned, ctx.positions,
+                       ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table, rank, self.rot_dim, write=cache.writes,
+                       query=query, query_head=self.kv_head, query_first=rank, source_head=self.q_head, source_first=self.dim,
+                       n_heads=heads)
         k.heads_linear(proj, self.q_head, 0, self.key_up, query, self.kv_head, 0, heads)
-        k.rotate_heads(proj, self.q_head, self.dim, query, self.kv_head, rank, self.frequencies, turned, ctx.positions,
-                       heads, self.rot_dim)
         attended = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
         k.attention(query, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions,
                     heads, 1, self.kv_head, self.scale, 0, layout=ctx)
-        values = ctx.new_activations(ctx.n_rows, heads * self.vdim)
+        values = ctx.new_activations(ctx.n_rows, heads * self.vdim, reader=self.out.reader())
         k.heads_linear(attended, self.kv_head, 0, self.value_up, values, self.vdim, 0, heads)
         self.out.forward(ctx, values, out=hidden, accumulate=not fresh)
         return None

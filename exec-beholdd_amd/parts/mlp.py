@@ -86,8 +86,9 @@ class SquaredReLU:
 
     def forward(self, ctx, x, hidden, fresh=False):
         inner = self.up.forward(ctx, x)
-        ctx.kernels.relu_squared(inner)
-        self.down.forward(ctx, inner, out=hidden, accumulate=not fresh)
+        activated = ctx.new_activations(inner.shape[0], self.inner, reader=self.down.reader())      # as the down product reads it
+        ctx.kernels.relu_squared(inner, activated)
+        self.down.forward(ctx, activated, out=hidden, accumulate=not fresh)
 
 
 @FEED_FORWARDS.register("squared_relu")

@@ -66,6 +66,16 @@ class ZeroCentredRMSNorm(RMSNorm):
         ctx.kernels.streams_rmsnorm(hidden, take, self.weight, self.eps, out, rows=rows)
         return out
 
+    def update_then_forward(self, ctx, hidden, result, mix, give, scale, reader=None, take=None):
+        """The streams' update by a sublayer's `result` (`kernels.streams_update`) and this norm of what they have become,
+        in one kernel; None where the kernel set has none (then update, and call `forward`)."""
+        fused = getattr(ctx.kernels, "streams_update_rmsnorm", None)
+        if fused is None or hidden.dim() != 3:
+            return None
+        out = ctx.new_activations(hidden.shape[0], self.width, reader=reader)
+        fused(hidden, result, mix, give, scale, take, self.weight, self.eps, out)
+        return out
+
     def request(self, reader=None):
         raise NotImplementedError("this norm does not ride on the products around it")
 

@@ -11,7 +11,8 @@ pre-norm residual X <- X + scale * F(norm(X)).  The model's output is the sum of
 forms (`ZeroCentredRMSNorm` reads [n, S, width] with every stream taken once).
 
 All of it is float32: the streams, their sums and the update.  The streams lie [rows, S, width]; two kernels do the
-work, `streams_rmsnorm` (sum, statistic and norm in one pass) and `streams_update`.  A sublayer that can write its
+work, `streams_rmsnorm` (sum, statistic and norm in one pass) and `streams_update`, and where another sublayer of
+this make follows (in this block or the next) one kernel does the update and that sublayer's norm together.  A sublayer that can write its
 result instead of adding it (`writes_fresh`) gets an empty matrix; any other registered mixer or feed-forward gets a
 zeroed one to add into, so the block takes every part the pre-norm block takes.
 """
@@ -126,29 +127,57 @@ class StreamMixingBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def _sublayer(self, ctx, hidden, norm, part, connection, *cache):
+    def _read(self, ctx, hidden, norm, part, connection):
         reader = getattr(part, "input_reader", None) if getattr(norm, "serves_reader", False) else None
         if getattr(norm, "reads_streams", False):
-            x = norm.forward(ctx, hidden, reader=reader, take=connection.take)
-        elif self.streams == 1 and connection.take is None:       # any other norm reads the one plain residual
+            return norm.forward(ctx, hidden, reader=reader, take=connection.take)
+        if self.streams == 1 and connection.take is None:       # any other norm reads the one plain residual
             plain = hidden.view(hidden.shape[0], self.width)
-            x = norm.forward(ctx, plain, reader=reader) if reader is not None else norm.forward(ctx, plain)
-        else:
-            raise TypeError(f"{type(norm).__name__} cannot read a weighted sum of residual streams")
+            return norm.forward(ctx, plain, reader=reader) if reader is not None else norm.forward(ctx, plain)
+        raise TypeError(f"{type(norm).__name__} cannot read a weighted sum of residual streams")
+
+    def _run(self, ctx, hidden, x, part, *cache):
         result = ctx.new_f32(hidden.shape[0], self.width)
         if getattr(part, "writes_fresh", False):
             part.forward(ctx, x, result, *cache, fresh=True)
         else:
             result.zero_()
             part.forward(ctx, x, result, *cache)
+        return result
+
+    @staticmethod
+    def _write(ctx, hidden, result, connection, then=None):
+        """The sublayer's result into the streams; `then` = (norm, part, connection) of the sublayer that runs next, whose
+        input the same kernel writes where norm and kernels offer it.  Returns that input, or None."""
+        if then is not None:
+            norm, part, following = then
+            fused = getattr(norm, "update_then_forward", None)
+            if fused is not None:
+                reader = getattr(part, "input_reader", None) if getattr(norm, "serves_reader", False) else None
+                x = fused(ctx, hidden, result, connection.mix, connection.give, connection.scale, reader=reader, take=following.take)
+                if x is not None:
+                    return x
         ctx.kernels.streams_update(hidden, result, connection.mix, connection.give, connection.scale)
+        return None
+
+    def entry(self):
+        """What the block before needs to prepare this block's first input: (norm, mixer, connection)."""
+        return (self.mixer_norm, self.mixer, self.mixer_connection)
 
     def forward(self, ctx, hidden, cache, prepared=None, next_block=None):
-        """`hidden` [rows, streams, width] float32, updated in place."""
-        self._sublayer(ctx, hidden, self.mixer_norm, self.mixer, self.mixer_connection, cache)
-        if self.feed_forward is not None:
-            self._sublayer(ctx, hidden, self.feed_forward_norm, self.feed_forward, self.feed_forward_connection)
-        return None
+        """`hidden` [rows, streams, width] float32, updated in place.  `prepared`: the mixer's input, if the block before
+        wrote it with its last update; returns the next block's, if this block could write it."""
+        following = next_block.entry() if isinstance(next_block, StreamMixingBlock) and next_block.streams == self.streams else None
+        x = prepared if prepared is not None else self._read(ctx, hidden, self.mixer_norm, self.mixer, self.mixer_connection)
+        result = self._run(ctx, hidden, x, self.mixer, cache)
+        if self.feed_forward is None:
+            return self._write(ctx, hidden, result, self.mixer_connection, following)
+        inner = (self.feed_forward_norm, self.feed_forward, self.feed_forward_connection)
+        x = self._write(ctx, hidden, result, self.mixer_connection, inner)
+        if x is None:
+            x = self._read(ctx, hidden, *inner)
+        result = self._run(ctx, hidden, x, self.feed_forward)
+        return self._write(ctx, hidden, result, self.feed_forward_connection, following)
 
 
 @BLOCKS.register("stream_mixing")

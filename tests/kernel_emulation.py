@@ -122,13 +122,17 @@ class TorchKernels:
         new = torch.einsum("st,nsd->ntd", m, x.double()) + g[None, :, None] * add[:, None, :]
         x.copy_(new.float())
 
+    def streams_update_rmsnorm(self, x, y, mix, give, scale, take, weight, eps, out):
+        self.streams_update(x, y, mix, give, scale)
+        self.streams_rmsnorm(x, take, weight, eps, out)
+
     def scale(self, x, factor):
         self.calls.append("scale")
         x.mul_(factor)
 
-    def relu_squared(self, x):
+    def relu_squared(self, x, out=None):
         self.calls.append("relu_squared")
-        x.copy_((x.float().clamp(min=0) ** 2).to(x.dtype))
+        (x if out is None else out).copy_((x.float().clamp(min=0) ** 2).to(x.dtype))
 
     # ---- linear attention with a decay ----
     def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
@@ -167,8 +171,12 @@ class TorchKernels:
         return torch.cat([a * c - b * s, b * c + a * s, rest], dim=-1)
 
     def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
-                     rank, rot_dim):
+                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0):
         self.calls.append("latent_write")
+        if query is not None:
+            self.rotate_heads(down, source_head, source_first, query, query_head, query_first, freq, turned, positions, n_heads, rot_dim)
+        if not write:
+            return
         x = down[:, offset:offset + rank + rot_dim].float()
         c = x[:, :rank] * (1.0 / torch.sqrt((x[:, :rank].double() ** 2).mean(-1, keepdim=True) + eps)).float()
         if weight is not None:
