@@ -173,7 +173,12 @@ def main(argv=None, stdin=None, stdout=None) -> int:
     from ..kernels import KernelError
     from ..kernels.build import BuildError
     try:
-        engine = Engine(args["--model"], dtype=args["--dtype"], max_tokens=args["--max-tokens"])
+        # --max-tokens counts the tokens that live requests hold, without padding; the cache hands out whole pages, and every
+        # live request may leave most of its last page unused: room for one more page for each of up to 64 live requests
+        # (never more requests than tokens).
+        from ..kernels.build import source_page_size
+        page = source_page_size()
+        engine = Engine(args["--model"], dtype=args["--dtype"], max_tokens=args["--max-tokens"] + page * min(64, args["--max-tokens"]))
         replayer = Replayer(engine, args["--out"], args["--capture"],
                             notes={"dtype": args["--dtype"], "max_tokens": args["--max-tokens"], "tool": "trace_run"})
     except (ValueError, OSError, CacheError, MemoryBudgetError, KernelError, BuildError) as error:

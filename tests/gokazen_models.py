@@ -121,3 +121,33 @@ def write_model(folder, config, weights):
     write_safetensors(os.path.join(folder, "model.safetensors"),
                       {name: torch.from_numpy(np.ascontiguousarray(value)).to(torch.bfloat16) for name, value in weights.items()})
     return str(folder)
+
+
+def drawn_config(seed):
+    """A configuration whose every size, count, constant and layer order is drawn: widths and head sizes that are no
+    multiples of 8 among them, one to four streams or none, a loop anywhere (also empty, also over everything)."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+    width = int(pick(24, 40, 52, 64, 72, 96, 130))
+    n_layers = int(rng.integers(1, 5))
+    layers = []
+    for index in range(n_layers):
+        ff = int(pick(0, 36, 64, 100))
+        if rng.random() < 0.5 or (index == n_layers - 1 and not any(l["type"] == "lightning" for l in layers) and rng.random() < 0.7):
+            heads = int(pick(1, 2, 3, 5))
+            layers.append(lightning(heads, int(pick(4, 12, 16, 33, 64)), int(pick(4, 10, 16, 40, 64, 72)),
+                                    [float(pick(0.3, 0.6, 0.9, 0.97, 0.999, 1.0)) for _ in range(heads)], ff=ff))
+        else:
+            rot_dim = int(pick(2, 4, 8, 16, 24))
+            dims = int(pick(*[d for d in (2, 4, 8, 16, 24) if d <= rot_dim]))
+            layers.append(latent(int(pick(1, 2, 3, 6)), int(pick(4, 8, 20, 32)), rot_dim, int(pick(4, 12, 16, 36)),
+                                 int(pick(8, 24, 30, 40, 56, 112)), float(pick(0.2, 0.35, 0.5, 1.0)),
+                                 base=float(pick(100.0, 10000.0, 500000.0)), dims=dims, ff=ff))
+    config = {"architecture": "Gokazen", "vocab": int(pick(37, 64, 150, 301)), "width": width,
+              "logit_scale": float(pick(0.25, 0.7, 1.0, 3.0)), "norm": {"eps": float(pick(1e-6, 1e-5, 1e-3))}, "layers": layers}
+    if rng.random() < 0.8:
+        config["streams"] = int(pick(1, 2, 3, 4))
+    if rng.random() < 0.8:
+        start = int(rng.integers(0, n_layers + 1))
+        config["loop"] = {"start": start, "stop": int(rng.integers(start, n_layers + 1)), "times": int(pick(1, 2, 3))}
+    return config

@@ -286,3 +286,18 @@ def test_prompts_longer_than_a_step_go_through_in_portions(folders):
     results = engine.generate(prompts, max_new_tokens=4)
     for prompt, result in zip(prompts, results):
         assert result.token_ids == plain.greedy(config, weights, prompt, 4)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations_on_the_torch_double(seed, tmp_path):
+    """Sizes, counts, constants and layer orders that nobody picked: whole prompts and a tail token by token."""
+    config = gm.drawn_config(seed)
+    folder = gm.write_model(tmp_path / "drawn", config, gm.random_weights(config, seed, gain=0.7))
+    _, weights = plain.load(folder)
+    requests = schedules.random_requests(config["vocab"], [1, 19, 70], seed=seed)
+    expected = [plain.forward(config, weights, r) for r in requests]
+    engine = make_engine(folder)
+    for label, got in (("whole", schedules.whole(engine, requests)), ("tail", schedules.tail_one_by_one(engine, requests, tail=5)),
+                       ("batches", schedules.batches(engine, requests, batch_size=3))):
+        for i, (g, e) in enumerate(zip(got, expected)):
+            assert schedules.relative_error(g, e) < 1e-4, (config, label, i, schedules.relative_error(g, e))
