@@ -14,7 +14,13 @@
 // with k'_j = decay^-(j+1) k_j and q'_t = decay^(t+1) q_t the inner loop is S' += k'_t v_t^T, o_t = S'^T q'_t, two
 // FMAs an element instead of three, and S' is scaled by decay^n once when the stage ends.  decay^-16 must stay a
 // modest number for that: heads that forget faster than 0.5 a row take the recurrence as written.
-// Steps of one row a sequence (decoding) are the same kernel: one stage of one row.
+// A long sequence that would leave compute units idle is cut into chunks of rows that are walked at the same time
+// (bh_lightning_chunks): every chunk but a sequence's first starts from a zero state and leaves its own end state in
+// scratch memory; lightning_combine_kernel then goes through a sequence's chunks in order, E_c = decay^rows_c E_(c-1) + Z_c,
+// leaves every chunk the state it should have started from and the cache the last one; and lightning_carry_kernel adds
+// what that state owes each row, decay^(t+1) E_(c-1)^T q_t (t counted from the chunk's first row), a small matrix product
+// per chunk and head.  All of it float32 FMA; the sums are the recurrence's, in another order.
+// Steps of one row a sequence (decoding) have a lean kernel of their own.
 #include "common.h"
 
 #define LN_TOKENS 16
@@ -30,11 +36,12 @@ template <typename T, int DPT, int VT>
 __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off,
                                       float* __restrict__ state, const float* __restrict__ decay,
                                       const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
-                                      float* __restrict__ out, int H, int dim, int vdim, int parts) {
+                                      float* __restrict__ out, int H, int dim, int vdim, int parts, int n_chunks,
+                                      int chunk_rows, float* __restrict__ chunk_state) {
   extern __shared__ __align__(16) float lds[];
   __shared__ float grow[LN_TOKENS], shrink[LN_TOKENS];      // decay^(t+1) and its inverse
   constexpr int PRE = (2 * LN_TOKENS * DPT + VT - 1) / VT + LN_TOKENS;      // a stage's elements a thread, at most
-  const int seq = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const int seq = blockIdx.x / n_chunks, chunk = blockIdx.x % n_chunks, head = blockIdx.y, tile = blockIdx.z;
   const int threads = blockDim.x;
   const int j = threadIdx.x % VT, part = threadIdx.x / VT;
   const int column = tile * VT + j;
@@ -43,7 +50,9 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
   float* ks = qs + LN_TOKENS * padded;            // [LN_TOKENS][padded]
   float* vs = ks + LN_TOKENS * padded;            // [LN_TOKENS][VT]
   float* sums = vs + LN_TOKENS * VT;              // [LN_TOKENS][parts][VT]
-  const int lo = seq_start[seq], hi = seq_start[seq + 1];
+  const int lo = seq_start[seq] + chunk * chunk_rows;
+  if (lo >= seq_start[seq + 1]) return;      // the sequence has no such chunk
+  const int hi = seq_start[seq + 1] < lo + chunk_rows ? seq_start[seq + 1] : lo + chunk_rows;
   const int slot = seq_slot[seq];
   const float lambda = decay[head];
   const bool scaled = lambda >= LN_SCALED_FROM;
@@ -54,12 +63,14 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
     shrink[threadIdx.x] = scaled ? 1.0f / power : 1.f;
   }
   float* mine = state + (((size_t)slot * H + head) * dim) * vdim;
+  // where the end state goes: the cache, or with chunks the chunk's place in scratch memory
+  float* left = n_chunks > 1 ? chunk_state + ((((size_t)seq * n_chunks + chunk) * H + head) * dim) * vdim : mine;
   const bool live = column < vdim;
   float s[DPT];
 #pragma unroll
   for (int e = 0; e < DPT; ++e) {
     const int i = part * DPT + e;
-    s[e] = (live && i < dim) ? mine[(size_t)i * vdim + column] : 0.f;
+    s[e] = (live && i < dim && chunk == 0) ? mine[(size_t)i * vdim + column] : 0.f;
   }
   // A stage's elements in one numbering, row after row: q [padded], k [padded], v [VT] of each row.  Where a thread's
   // elements come from (the column of a projected row, -1 for padding) and go to (the place in LDS) is worked out
@@ -174,7 +185,7 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
 #pragma unroll
     for (int e = 0; e < DPT; ++e) {
       const int i = part * DPT + e;
-      if (i < dim) mine[(size_t)i * vdim + column] = s[e];
+      if (i < dim) left[(size_t)i * vdim + column] = s[e];
     }
   }
 }
@@ -236,16 +247,102 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_step_kernel(
   }
 }
 
+// The chunks of a sequence in order (see the top of the file): a thread an element of the state.
+__global__ __launch_bounds__(256) void lightning_combine_kernel(float* __restrict__ chunk_state, float* __restrict__ state,
+                                                                const float* __restrict__ decay,
+                                                                const int32_t* __restrict__ seq_start,
+                                                                const int32_t* __restrict__ seq_slot, int H, int size,
+                                                                int n_chunks, int chunk_rows) {
+  const int seq = blockIdx.x, head = blockIdx.y, at = blockIdx.z * 256 + threadIdx.x;
+  if (at >= size) return;
+  const int rows = seq_start[seq + 1] - seq_start[seq];
+  if (rows <= 0) return;
+  const float lambda = decay[head];
+  const size_t apart = (size_t)H * size;
+  float* z = chunk_state + ((size_t)seq * n_chunks * H + head) * size + at;
+  float end = z[0];
+  for (int c = 1; c * chunk_rows < rows; ++c) {
+    const int here = rows - c * chunk_rows < chunk_rows ? rows - c * chunk_rows : chunk_rows;
+    const float own = z[c * apart];
+    z[c * apart] = end;      // what chunk c should have started from
+    end = fmaf(powf(lambda, (float)here), end, own);
+  }
+  state[((size_t)seq_slot[seq] * H + head) * size + at] = end;
+}
+
+// out[row] += decay^(t+1) E^T silu(q[row]) for the rows of every chunk but a sequence's first, E the state the chunk
+// should have started from: LC_ROWS rows of one chunk and head a workgroup, their queries through LDS, a thread a
+// value column.
+#define LC_ROWS 16
+template <typename T>
+__global__ __launch_bounds__(256) void lightning_carry_kernel(const T* __restrict__ proj, int row_stride, int q_off,
+                                                              const float* __restrict__ chunk_state,
+                                                              const float* __restrict__ decay,
+                                                              const int32_t* __restrict__ seq_start, float* __restrict__ out,
+                                                              int H, int dim, int vdim, int n_chunks, int chunk_rows) {
+  extern __shared__ __align__(16) float xs[];      // [dim][LC_ROWS]
+  const int per_chunk = chunk_rows / LC_ROWS;
+  const int piece = blockIdx.x % per_chunk, chunk = 1 + (blockIdx.x / per_chunk) % (n_chunks - 1);
+  const int seq = blockIdx.x / (per_chunk * (n_chunks - 1)), head = blockIdx.y;
+  const int first = seq_start[seq] + chunk * chunk_rows, lo = first + piece * LC_ROWS;
+  const int last = seq_start[seq + 1] < first + chunk_rows ? seq_start[seq + 1] : first + chunk_rows;
+  if (lo >= last) return;
+  const int rows = last - lo < LC_ROWS ? last - lo : LC_ROWS;
+  const float lambda = decay[head];
+  for (int e = threadIdx.x; e < dim * LC_ROWS; e += blockDim.x) {
+    const int i = e / LC_ROWS, r = e % LC_ROWS;
+    float value = 0.f;
+    if (r < rows)
+      value = silu_f32(to_f32(proj[(size_t)(lo + r) * row_stride + q_off + (size_t)head * dim + i])) *
+              powf(lambda, (float)(piece * LC_ROWS + r + 1));
+    xs[e] = value;
+  }
+  __syncthreads();
+  const int column = blockIdx.z * blockDim.x + threadIdx.x;
+  if (column >= vdim) return;
+  const float* from = chunk_state + ((((size_t)seq * n_chunks + chunk) * H + head) * dim) * vdim + column;
+  float acc[LC_ROWS] = {};
+  for (int i = 0; i < dim; ++i) {
+    const float w = from[(size_t)i * vdim];
+#pragma unroll
+    for (int r = 0; r < LC_ROWS; r += 4) {
+      const float4 x4 = *reinterpret_cast<const float4*>(xs + i * LC_ROWS + r);
+      acc[r] = fmaf(x4.x, w, acc[r]);
+      acc[r + 1] = fmaf(x4.y, w, acc[r + 1]);
+      acc[r + 2] = fmaf(x4.z, w, acc[r + 2]);
+      acc[r + 3] = fmaf(x4.w, w, acc[r + 3]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < LC_ROWS; ++r)
+    if (r < rows) out[((size_t)(lo + r) * H + head) * vdim + column] += acc[r];
+}
+
+// Into how many chunks of how many rows the sequences of a step are cut (1: not at all): as many as it takes to give
+// every compute unit two workgroups of 64 value columns, chunks of 64 rows at least and whole stages of rows.
+extern "C" int bh_lightning_chunks(int n_seqs, int n_rows, int max_rows, int H, int vdim, int* chunk_rows) {
+  const int tiles = (vdim + 63) / 64;
+  const long groups = (long)n_seqs * H * tiles, wanted = 2L * bh_compute_units();
+  *chunk_rows = max_rows > 0 ? max_rows : 1;
+  if (n_rows == n_seqs || max_rows < 128 || groups >= wanted) return 1;
+  const long cuts = (wanted + groups - 1) / groups;
+  int rows = (int)((max_rows + cuts - 1) / cuts);
+  rows = rows < 64 ? 64 : (rows + LN_TOKENS - 1) / LN_TOKENS * LN_TOKENS;
+  *chunk_rows = rows;
+  return (max_rows + rows - 1) / rows;
+}
+
 template <typename T, int DPT, int VT>
 static int launch_lightning(const void* proj, int row_stride, int q_off, int k_off, int v_off, float* state,
                             const float* decay, const int32_t* seq_start, const int32_t* seq_slot, float* out, int n_seqs,
-                            int n_rows, int H, int dim, int vdim, hipStream_t stream) {
+                            int n_rows, int H, int dim, int vdim, int n_chunks, int chunk_rows, float* chunk_state,
+                            hipStream_t stream) {
   const int parts = (dim + DPT - 1) / DPT;
   BH_REQUIRE(parts * VT <= 1024, "lightning: heads of %d x %d need more than 1024 threads", dim, vdim);
   const int tiles = (vdim + VT - 1) / VT;
   const size_t smem = (size_t)LN_TOKENS * (2 * parts * DPT + VT + parts * VT) * sizeof(float);
   BH_REQUIRE(smem <= 63 * 1024, "lightning: heads of %d x %d need %zu bytes of LDS", dim, vdim, smem);
-  dim3 grid(n_seqs, H, tiles), block(parts * VT);
+  dim3 grid(n_seqs * n_chunks, H, tiles), block(parts * VT);
   if (n_rows == n_seqs) {      // one row each
     const size_t lean = (size_t)(2 * parts * DPT + VT + parts * VT) * sizeof(float);
     lightning_step_kernel<T, DPT, VT><<<grid, block, lean, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, state, decay,
@@ -253,8 +350,19 @@ static int launch_lightning(const void* proj, int row_stride, int q_off, int k_o
     return bh_check_launch("lightning_step");
   }
   lightning_scan_kernel<T, DPT, VT><<<grid, block, smem, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, state, decay,
-                                                                   seq_start, seq_slot, out, H, dim, vdim, parts);
-  return bh_check_launch("lightning_scan");
+                                                                   seq_start, seq_slot, out, H, dim, vdim, parts, n_chunks,
+                                                                   chunk_rows, chunk_state);
+  if (int status = bh_check_launch("lightning_scan")) return status;
+  if (n_chunks == 1) return 0;
+  const int size = dim * vdim;
+  lightning_combine_kernel<<<dim3(n_seqs, H, (size + 255) / 256), dim3(256), 0, stream>>>(chunk_state, state, decay, seq_start,
+                                                                                          seq_slot, H, size, n_chunks, chunk_rows);
+  if (int status = bh_check_launch("lightning_combine")) return status;
+  const int columns = vdim >= 256 ? 256 : (vdim + 63) / 64 * 64;
+  dim3 carry(n_seqs * (n_chunks - 1) * (chunk_rows / LC_ROWS), H, (vdim + columns - 1) / columns);
+  lightning_carry_kernel<T><<<carry, dim3(columns), (size_t)dim * LC_ROWS * sizeof(float), stream>>>(
+      (const T*)proj, row_stride, q_off, chunk_state, decay, seq_start, out, H, dim, vdim, n_chunks, chunk_rows);
+  return bh_check_launch("lightning_carry");
 }
 
 // proj [n_rows][row_stride]: a row holds q (H x dim) from q_off, k (H x dim) from k_off, v (H x vdim) from v_off, all
@@ -262,7 +370,8 @@ static int launch_lightning(const void* proj, int row_stride, int q_off, int k_o
 // sequence in slot seq_slot[b], in order, and every sequence has at least one.  out [n_rows][H * vdim] float32.
 extern "C" int bh_lightning_scan(const void* proj, int dtype, int row_stride, int q_off, int k_off, int v_off, float* state,
                                  const float* decay, const int32_t* seq_start, const int32_t* seq_slot, float* out,
-                                 int n_seqs, int n_rows, int H, int dim, int vdim, hipStream_t stream) {
+                                 int n_seqs, int n_rows, int max_rows, int H, int dim, int vdim, float* chunk_state,
+                                 long chunk_state_floats, hipStream_t stream) {
   BH_REQUIRE(n_seqs > 0 && n_rows >= n_seqs && H > 0 && dim > 0 && vdim > 0,
              "lightning: sizes must be positive, and every sequence of the step brings a row");
   BH_REQUIRE(H <= 65535 && n_seqs <= 2147483647, "lightning: too many heads");
@@ -270,15 +379,22 @@ extern "C" int bh_lightning_scan(const void* proj, int dtype, int row_stride, in
   BH_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + H * dim <= row_stride && k_off + H * dim <= row_stride &&
                  v_off + H * vdim <= row_stride,
              "lightning: q, k and v do not lie inside a row of %d", row_stride);
+  // max_rows: no sequence of the step brings more rows (what the cut into chunks is made for)
+  int chunk_rows = 0;
+  const int n_chunks = bh_lightning_chunks(n_seqs, n_rows, max_rows > 0 && max_rows < n_rows ? max_rows : n_rows, H, vdim, &chunk_rows);
+  BH_REQUIRE(n_chunks == 1 || (chunk_state != nullptr && chunk_state_floats >= (long)n_seqs * n_chunks * H * dim * vdim),
+             "lightning: %d chunks a sequence need scratch memory for their states", n_chunks);
+  BH_REQUIRE((long)n_seqs * n_chunks * (chunk_rows / LC_ROWS + 1) < (1L << 31), "lightning: too many workgroups");
+  BH_REQUIRE((size_t)dim * LC_ROWS * sizeof(float) <= 63 * 1024, "lightning: a key size of %d is too large to cut a sequence into chunks", dim);
   // value columns a workgroup: 64 where that many workgroups fill the chip twice, else fewer, down to 16
   int vt = vdim > 32 ? 64 : (vdim > 16 ? 32 : 16);
-  while (vt > 16 && (long)n_seqs * H * ((vdim + vt - 1) / vt) < 2L * bh_compute_units()) vt /= 2;
+  while (vt > 16 && (long)n_seqs * n_chunks * H * ((vdim + vt - 1) / vt) < 2L * bh_compute_units()) vt /= 2;
   const int slice = (dim + 256 / vt - 1) / (256 / vt);      // slices of dim that make the workgroup four waves
 #define BH_LN(T, DPT)                                                                                                   \
   do {                                                                                                                  \
-    if (vt == 64) return launch_lightning<T, DPT, 64>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
-    if (vt == 32) return launch_lightning<T, DPT, 32>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
-    return launch_lightning<T, DPT, 16>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, stream); \
+    if (vt == 64) return launch_lightning<T, DPT, 64>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, n_chunks, chunk_rows, chunk_state, stream); \
+    if (vt == 32) return launch_lightning<T, DPT, 32>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, n_chunks, chunk_rows, chunk_state, stream); \
+    return launch_lightning<T, DPT, 16>(proj, row_stride, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_seqs, n_rows, H, dim, vdim, n_chunks, chunk_rows, chunk_state, stream); \
   } while (0)
 #define BH_LN_SIZES(T)            \
   if (slice <= 4) BH_LN(T, 4);    \

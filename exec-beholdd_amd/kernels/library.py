@@ -167,7 +167,8 @@ class KernelSizes:
             "bh_streams_update_rmsnorm": [p, p, p, p, p, p, p, p, i, i, i, i, f, i, p],
             "bh_scale": [p, ctypes.c_long, f, p],
             "bh_relu_squared": [p, p, i, i, i, i, p],
-            "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, i, p],
+            "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, p],
+            "bh_lightning_chunks": [i, i, i, i, i, p],
             "bh_gated_rmsnorm": [p, p, i, i, p, p, i, i, f, i, p],
             "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, i, i, i, i, i, p],
             "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, i, p],
@@ -819,10 +820,20 @@ class HipKernels(KernelSizes):
                                              _code(x, "relu_squared x"), x.shape[0], x.shape[1], _block_rows(out), self._stream()))
 
     # ---- linear attention with a decay, as a recurrence over a float32 state ----
-    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
+    def lightning_chunk_bytes(self, n_seqs, n_rows, max_rows, n_heads, dim, vdim) -> int:
+        """Bytes of scratch memory that `lightning_scan` allocates for a step of these sizes (the states of the chunks it cuts
+        long sequences into)."""
+        rows = ctypes.c_int(0)
+        chunks = int(self.lib.bh_lightning_chunks(int(n_seqs), int(n_rows), int(max_rows), int(n_heads), int(vdim), ctypes.byref(rows)))
+        return _rounded(n_seqs * chunks * n_heads * dim * vdim * 4) if chunks > 1 else 0
+
+    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim,
+                       max_rows_per_seq=None):
         """For every sequence b of the step (rows seq_start[b] .. seq_start[b + 1] - 1 in order, state row seq_slot[b]) and
         head h: S <- decay[h] * S + k_t v_t^T, out_t = S^T q_t with q, k, v = silu of the row's slices from q_off, k_off,
-        v_off of `proj` [n, P].  state f32 [slots, H, dim, vdim] in place, out f32 [n, H * vdim]."""
+        v_off of `proj` [n, P].  state f32 [slots, H, dim, vdim] in place, out f32 [n, H * vdim].  `max_rows_per_seq`: no
+        sequence of the step brings more rows (the step's total, if it is not given); long sequences that would leave the
+        chip idle are cut into chunks that run side by side, whose states take scratch memory for the length of the call."""
         n_rows, stride = proj.shape
         n_seqs = seq_slot.shape[0]
         if (state.dim() != 4 or tuple(state.shape[1:]) != (n_heads, dim, vdim) or tuple(out.shape) != (n_rows, n_heads * vdim)
@@ -830,11 +841,16 @@ class HipKernels(KernelSizes):
             raise KernelError(f"lightning_scan: shapes proj {tuple(proj.shape)}, state {tuple(state.shape)}, out "
                               f"{tuple(out.shape)} do not fit {n_heads} heads of {dim} x {vdim} and {n_seqs} sequences")
         f32, i32 = (torch.float32,), (torch.int32,)
+        most = min(int(max_rows_per_seq), n_rows) if max_rows_per_seq else n_rows
+        chunk_rows = ctypes.c_int(0)
+        chunks = int(self.lib.bh_lightning_chunks(n_seqs, n_rows, most, n_heads, vdim, ctypes.byref(chunk_rows)))
+        scratch = torch.empty(n_seqs * chunks * n_heads * dim * vdim, dtype=torch.float32, device=self.device) if chunks > 1 else None
         self._check(self.lib.bh_lightning_scan(
             self._ptr(proj, "lightning proj"), _code(proj, "lightning proj"), stride, int(q_off), int(k_off), int(v_off),
             self._ptr(state, "lightning state", f32), self._ptr(decay, "lightning decay", f32),
             self._ptr(seq_start, "seq_start", i32), self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "lightning out", f32),
-            n_seqs, n_rows, n_heads, dim, vdim, self._stream()))
+            n_seqs, n_rows, most, n_heads, dim, vdim, self._ptr(scratch, "chunk states", f32, True),
+            scratch.numel() if scratch is not None else 0, self._stream()))
 
     def gated_rmsnorm(self, o, proj, gate_off, weight, eps, out):
         """out[r] = RMSNorm(o[r]) * weight * sigmoid(proj[r, gate_off : gate_off + W]); o f32 [n, W], out [n, W] in the

@@ -62,7 +62,10 @@ class LightningAttention:
 
     def working_bytes(self, step) -> int:
         width = self.n_heads * self.vdim
-        return (self.proj.working_bytes(step, step.rows) + step.matrix(step.rows, width, 4)
+        chunks = 0
+        if step.sizes is not None and hasattr(step.sizes, "lightning_chunk_bytes"):
+            chunks = step.sizes.lightning_chunk_bytes(step.seqs, step.rows, step.max_rows_per_seq, self.n_heads, self.dim, self.vdim)
+        return (chunks + self.proj.working_bytes(step, step.rows) + step.matrix(step.rows, width, 4)
                 + step.matrix(step.rows, width, reader=self.out.reader_for_plan(step.act_size))
                 + self.out.working_bytes(step, step.rows, accumulate=True))
 
@@ -72,7 +75,7 @@ class LightningAttention:
         proj = self.proj.forward(ctx, x)
         mixed = ctx.new_f32(ctx.n_rows, width)
         k.lightning_scan(proj, self.q_off, self.k_off, self.v_off, cache.state, self.decay, ctx.seq_start, ctx.seq_slot,
-                         mixed, self.n_heads, self.dim, self.vdim)
+                         mixed, self.n_heads, self.dim, self.vdim, max_rows_per_seq=ctx.max_rows_per_seq)
         gated = ctx.new_activations(ctx.n_rows, width, reader=self.out.reader())
         k.gated_rmsnorm(mixed, proj, self.g_off, self.norm_weight, self.norm_eps, gated)
         self.out.forward(ctx, gated, out=hidden, accumulate=not fresh)

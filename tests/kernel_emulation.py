@@ -135,7 +135,8 @@ class TorchKernels:
         (x if out is None else out).copy_((x.float().clamp(min=0) ** 2).to(x.dtype))
 
     # ---- linear attention with a decay ----
-    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim):
+    def lightning_scan(self, proj, q_off, k_off, v_off, state, decay, seq_start, seq_slot, out, n_heads, dim, vdim,
+                       max_rows_per_seq=None):
         self.calls.append("lightning_scan")
         silu = lambda z: z / (1 + torch.exp(-z))
         p = proj.float()

@@ -112,6 +112,9 @@ def test_small_elementwise_kernels(K, dtype):
     (3, 20, 12, [0.99, 0.9, 0.7], [33, 2, 2, 16]),      # sizes that are no power of two
     (2, 128, 128, [0.99, 0.95], [70]),                  # the sizes of a large model's heads: two value tiles
     (1, 200, 72, [0.98], [19]),                         # a key size whose slices are padded
+    (2, 16, 24, [0.9, 0.999], [700, 3, 130]),           # long enough to be cut into chunks that run side by side; a short one beside
+    (2, 128, 128, [0.995, 0.4], [333]),                 # chunks whose last one is not full; a head that forgets fast
+    (3, 40, 40, [1.0, 0.97, 0.6], [129, 64, 65, 128]),  # sequences that end at, before and after a chunk's end
 ])
 def test_lightning_scan(K, dtype, heads, dim, vdim, decay, lengths):
     """The recurrence over ragged rows of several sequences, into slots in another order than the batch's, and then
@@ -130,7 +133,7 @@ def test_lightning_scan(K, dtype, heads, dim, vdim, decay, lengths):
         starts = np.concatenate([[0], np.cumsum(lengths_now)]).astype(np.int32)
         out = torch.empty(n, values, device="cuda:0")
         K.lightning_scan(dev(t), q_off, k_off, v_off, state, dev(np.asarray(decay, np.float32)), dev(starts),
-                         dev(np.asarray(slots, np.int32)), out, heads, dim, vdim)
+                         dev(np.asarray(slots, np.int32)), out, heads, dim, vdim, max_rows_per_seq=max(lengths_now))
         for b, slot in enumerate(slots):
             rows = proj[starts[b]:starts[b + 1]]
             q = plain.silu(rows[:, q_off:q_off + keys]).reshape(-1, heads, dim).astype(np.float64)
