@@ -104,21 +104,19 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
     const int t = tok[i] < LN_TOKENS ? tok[i] : 0;
     mul[i] = dst[i] < q_end ? grow[t] : (dst[i] < k_end ? shrink[t] : 1.f);
   }
-  float raw[PRE];
+  // What a load brings stays as it came until the stage is written into LDS: nothing in `fetch` reads a loaded value
+  // (its widening to float32 and its mask come in `stage`), or every load would be waited for before the next is issued.
+  T raw[PRE];
   auto fetch = [&](int r0) {
     const int n = hi - r0 < LN_TOKENS ? hi - r0 : LN_TOKENS;
     const T* first = proj + (size_t)r0 * row_stride;
 #pragma unroll
-    for (int i = 0; i < PRE; ++i) {
-      const bool there = tok[i] < n && src[i] >= 0;
-      const float value = to_f32(first[there ? src[i] : 0]);
-      raw[i] = there ? value : 0.f;
-    }
+    for (int i = 0; i < PRE; ++i) raw[i] = first[(tok[i] < n && src[i] >= 0) ? src[i] : 0];
   };
   auto stage = [&](int n) {
 #pragma unroll
     for (int i = 0; i < PRE; ++i) {
-      if (i < pre && tok[i] < n) lds[dst[i]] = silu_f32(raw[i]) * mul[i];
+      if (i < pre && tok[i] < n) lds[dst[i]] = src[i] >= 0 ? silu_f32(to_f32(raw[i])) * mul[i] : 0.f;
     }
   };
   if (lo < hi) fetch(lo);
@@ -128,11 +126,13 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
     stage(n);
     __syncthreads();
     if (r0 + LN_TOKENS < hi) fetch(r0 + LN_TOKENS);      // on its way while this stage is computed
+    // (The row's sum over this thread's slice is returned, not stored: a store into LDS between two rows' reads of LDS
+    // would keep the next row's reads from starting early.  Two running sums halve the chain of dependent FMAs.)
     auto row_scaled = [&](int t) {
       const float v = vs[t * VT + j];
       const float* kt = ks + t * padded + part * DPT;
       const float* qt = qs + t * padded + part * DPT;
-      float acc = 0.f;
+      float even = 0.f, odd = 0.f;
 #pragma unroll
       for (int e = 0; e < DPT; e += 4) {
         const float4 k4 = *reinterpret_cast<const float4*>(kt + e), q4 = *reinterpret_cast<const float4*>(qt + e);
@@ -140,12 +140,12 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
         s[e + 1] = fmaf(k4.y, v, s[e + 1]);
         s[e + 2] = fmaf(k4.z, v, s[e + 2]);
         s[e + 3] = fmaf(k4.w, v, s[e + 3]);
-        acc = fmaf(s[e], q4.x, acc);
-        acc = fmaf(s[e + 1], q4.y, acc);
-        acc = fmaf(s[e + 2], q4.z, acc);
-        acc = fmaf(s[e + 3], q4.w, acc);
+        even = fmaf(s[e], q4.x, even);
+        odd = fmaf(s[e + 1], q4.y, odd);
+        even = fmaf(s[e + 2], q4.z, even);
+        odd = fmaf(s[e + 3], q4.w, odd);
       }
-      sums[(t * parts + part) * VT + j] = acc;
+      return even + odd;
     };
     auto row_plain = [&](int t) {
       const float v = vs[t * VT + j];
@@ -160,11 +160,14 @@ __global__ __launch_bounds__(DPT == 64 ? 1024 : 256) void lightning_scan_kernel(
       sums[(t * parts + part) * VT + j] = acc;
     };
     if (scaled) {
-      if (n == LN_TOKENS) {      // a whole stage: a trip count the compiler knows, so that it reads rows ahead
-#pragma unroll 4
-        for (int t = 0; t < LN_TOKENS; ++t) row_scaled(t);
+      if (n == LN_TOKENS) {      // a whole stage: every row's reads can start before the row before is done
+        float row_sums[LN_TOKENS];
+#pragma unroll
+        for (int t = 0; t < LN_TOKENS; ++t) row_sums[t] = row_scaled(t);
+#pragma unroll
+        for (int t = 0; t < LN_TOKENS; ++t) sums[(t * parts + part) * VT + j] = row_sums[t];
       } else {
-        for (int t = 0; t < n; ++t) row_scaled(t);
+        for (int t = 0; t < n; ++t) sums[(t * parts + part) * VT + j] = row_scaled(t);
       }
       const float back = grow[n - 1];
 #pragma unroll
@@ -302,6 +305,7 @@ __global__ __launch_bounds__(256) void lightning_carry_kernel(const T* __restric
   if (column >= vdim) return;
   const float* from = chunk_state + ((((size_t)seq * n_chunks + chunk) * H + head) * dim) * vdim + column;
   float acc[LC_ROWS] = {};
+#pragma unroll 8      // eight elements of the state asked for before the first is used
   for (int i = 0; i < dim; ++i) {
     const float w = from[(size_t)i * vdim];
 #pragma unroll
