@@ -1261,7 +1261,7 @@ def test_kernels_refuse_what_they_cannot_do(K):
     with pytest.raises(KernelError):
         K.rmsnorm(x, torch.ones(7, device="cuda:0"), 1e-6, torch.zeros(2, 8, device="cuda:0"))
     with pytest.raises(KernelError):      # a head size above the attention kernels' limit
-        hd = 512
+        hd = 1056
         K.attention(torch.zeros(1, hd, device="cuda:0"), torch.zeros(1, hd, device="cuda:0"),
                     torch.zeros(1, 1, PAGE, hd, device="cuda:0"), torch.zeros(1, 1, hd, PAGE, device="cuda:0"),
                     torch.zeros(1, 1, dtype=torch.int32, device="cuda:0"), torch.zeros(1, dtype=torch.int32, device="cuda:0"),
