@@ -301,3 +301,18 @@ def test_drawn_configurations_on_the_torch_double(seed, tmp_path):
                        ("batches", schedules.batches(engine, requests, batch_size=3))):
         for i, (g, e) in enumerate(zip(got, expected)):
             assert schedules.relative_error(g, e) < 1e-4, (config, label, i, schedules.relative_error(g, e))
+
+
+def test_the_command_line_plans_the_bytes_of_this_design_without_a_gpu(folders):
+    import io
+    from beholdd import cli
+    folder, _ = folders("deep")
+    out = io.StringIO()
+    code = cli.main(["generate", "--model", folder, "--prompt-ids", "1,2,3", "--max-new-tokens", "70", "--dtype", "bfloat16",
+                     "--plan-only"], out=out)
+    text = out.getvalue()
+    assert code == 0, text
+    # four runs of latent layers (two kinds of cached head) and four of lightning layers (two kinds of state)
+    assert "keys/values of 1 layers (1 heads x 128)" in text and "keys/values of 3 layers (1 heads x 64)" in text
+    assert "state (2, 64, 32) of 3 layers" in text and "state (4, 32, 48) of 1 layers" in text
+    assert "not counted" not in text          # every part says what a step of its allocates
