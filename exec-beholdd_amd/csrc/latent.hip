@@ -115,12 +115,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__ x, long x_row, int x_head, int x_first,
                                                            const T* __restrict__ w, T* __restrict__ y, long y_row, int y_head,
                                                            int y_first, int n_rows, int n_in, int n_out, int y_block_rows) {
-  extern __shared__ float xs[];      // [HL_ROWS][n_in]
+  extern __shared__ __align__(16) float xs[];      // [n_in][HL_ROWS]: the rows' values of one input side by side
   const int row0 = blockIdx.x * HL_ROWS, head = blockIdx.y, o = blockIdx.z * 256 + threadIdx.x;
   const int rows = n_rows - row0 < HL_ROWS ? n_rows - row0 : HL_ROWS;
   for (int e = threadIdx.x; e < HL_ROWS * n_in; e += 256) {
-    const int r = e / n_in, i = e % n_in;
-    xs[e] = r < rows ? to_f32(x[(size_t)(row0 + r) * x_row + (size_t)head * x_head + x_first + i]) : 0.f;
+    const int r = e / n_in, i = e % n_in;      // neighbouring threads read neighbouring inputs of a row
+    xs[i * HL_ROWS + r] = r < rows ? to_f32(x[(size_t)(row0 + r) * x_row + (size_t)head * x_head + x_first + i]) : 0.f;
   }
   __syncthreads();
   if (o >= n_out) return;
@@ -129,7 +129,13 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__
   for (int i = 0; i < n_in; ++i) {
     const float wv = to_f32(wh[(size_t)i * n_out]);
 #pragma unroll
-    for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(xs[r * n_in + i], wv, acc[r]);
+    for (int r = 0; r < HL_ROWS; r += 4) {      // four rows a read of LDS, the same address for every lane
+      const float4 x4 = *reinterpret_cast<const float4*>(xs + i * HL_ROWS + r);
+      acc[r] = fmaf(x4.x, wv, acc[r]);
+      acc[r + 1] = fmaf(x4.y, wv, acc[r + 1]);
+      acc[r + 2] = fmaf(x4.z, wv, acc[r + 2]);
+      acc[r + 3] = fmaf(x4.w, wv, acc[r + 3]);
+    }
   }
 #pragma unroll
   for (int r = 0; r < HL_ROWS; ++r)
