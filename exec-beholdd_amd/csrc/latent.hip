@@ -142,6 +142,49 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const T* __restrict__
     if (r < rows) y[bh_rows_index(y_block_rows, row0 + r, head * y_head + y_first + o, (int)y_row)] = from_f32<T>(acc[r]);
 }
 
+// The same for a step of at most HL_ROWS rows (decoding): a workgroup takes 64 outputs of one head and its four waves
+// a quarter of the inputs each, so that a head's weights are streamed by several workgroups and no thread walks all the
+// inputs alone; the quarters' sums are added through LDS in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(256) void heads_linear_few_kernel(const T* __restrict__ x, long x_row, int x_head, int x_first,
+                                                               const T* __restrict__ w, T* __restrict__ y, long y_row, int y_head,
+                                                               int y_first, int n_rows, int n_in, int n_out, int y_block_rows) {
+  extern __shared__ __align__(16) float xs[];      // [n_in][HL_ROWS]
+  __shared__ float parts[3][64][HL_ROWS + 1];
+  const int head = blockIdx.y, lane = threadIdx.x % 64, quarter = threadIdx.x / 64, o = blockIdx.z * 64 + lane;
+  for (int e = threadIdx.x; e < HL_ROWS * n_in; e += 256) {
+    const int r = e / n_in, i = e % n_in;
+    xs[i * HL_ROWS + r] = r < n_rows ? to_f32(x[(size_t)r * x_row + (size_t)head * x_head + x_first + i]) : 0.f;
+  }
+  __syncthreads();
+  const int each = (n_in + 3) / 4, from = quarter * each, to = from + each < n_in ? from + each : n_in;
+  const T* wh = w + (size_t)head * n_in * n_out + (o < n_out ? o : n_out - 1);
+  float acc[HL_ROWS] = {};
+  for (int i = from; i < to; ++i) {
+    const float wv = to_f32(wh[(size_t)i * n_out]);
+#pragma unroll
+    for (int r = 0; r < HL_ROWS; r += 4) {
+      const float4 x4 = *reinterpret_cast<const float4*>(xs + i * HL_ROWS + r);
+      acc[r] = fmaf(x4.x, wv, acc[r]);
+      acc[r + 1] = fmaf(x4.y, wv, acc[r + 1]);
+      acc[r + 2] = fmaf(x4.z, wv, acc[r + 2]);
+      acc[r + 3] = fmaf(x4.w, wv, acc[r + 3]);
+    }
+  }
+  if (quarter > 0) {
+#pragma unroll
+    for (int r = 0; r < HL_ROWS; ++r) parts[quarter - 1][lane][r] = acc[r];
+  }
+  __syncthreads();
+  if (quarter > 0 || o >= n_out) return;
+#pragma unroll
+  for (int r = 0; r < HL_ROWS; ++r) {
+    if (r >= n_rows) continue;
+    const float total = ((acc[r] + parts[0][lane][r]) + parts[1][lane][r]) + parts[2][lane][r];
+    y[bh_rows_index(y_block_rows, r, head * y_head + y_first + o, (int)y_row)] = from_f32<T>(total);
+  }
+}
+
 extern "C" int bh_heads_linear(const void* x, long x_row, int x_head, int x_first, const void* w, void* y, long y_row,
                                int y_head, int y_first, int dtype, int n_rows, int H, int n_in, int n_out, int y_block_rows,
                                hipStream_t stream) {
@@ -155,6 +198,17 @@ extern "C" int bh_heads_linear(const void* x, long x_row, int x_head, int x_firs
              "heads_linear: the heads' slices do not lie inside their rows");
   const size_t smem = (size_t)HL_ROWS * n_in * sizeof(float);
   BH_REQUIRE(smem <= 64 * 1024, "heads_linear: %d inputs a head are above the limit of %d", n_in, 64 * 1024 / 4 / HL_ROWS);
+  if (n_rows <= HL_ROWS && smem + sizeof(float) * 3 * 64 * (HL_ROWS + 1) <= 64 * 1024) {      // (its partial sums need LDS too)
+    dim3 few(1, H, (n_out + 63) / 64);
+#define BH_HL_FEW(T)                                                                                                      \
+  heads_linear_few_kernel<T><<<few, dim3(256), smem, stream>>>((const T*)x, x_row, x_head, x_first, (const T*)w, (T*)y, y_row, \
+                                                               y_head, y_first, n_rows, n_in, n_out, y_block_rows)
+    if (dtype == BH_F32) BH_HL_FEW(float);
+    else if (dtype == BH_BF16) BH_HL_FEW(bf16_t);
+    else return bh_fail("heads_linear: unknown dtype %d", dtype);
+#undef BH_HL_FEW
+    return bh_check_launch("heads_linear_few");
+  }
   dim3 grid((n_rows + HL_ROWS - 1) / HL_ROWS, H, (n_out + 255) / 256), block(256);
 #define BH_HL(T)                                                                                                         \
   heads_linear_kernel<T><<<grid, block, smem, stream>>>((const T*)x, x_row, x_head, x_first, (const T*)w, (T*)y, y_row, y_head, \
