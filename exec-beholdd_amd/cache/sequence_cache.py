@@ -69,8 +69,9 @@ class CachePlan:
         for g in self.groups:
             if g.need.kind == "kv":
                 window = f", window {g.need.window}" if g.need.window else ""
+                beside = f", and a state {tuple(g.need.state_shape)}: {g.state_bytes} bytes" if g.need.state_shape else ""
                 lines.append(f"  keys/values of {len(g.entries)} layers ({g.need.kv_heads} heads x "
-                             f"{g.need.head_dim}{window}): {g.kv_bytes} bytes")
+                             f"{g.need.head_dim}{window}): {g.kv_bytes} bytes{beside}")
             else:
                 lines.append(f"  state {tuple(g.need.state_shape)} of {len(g.entries)} layers: {g.state_bytes} bytes")
         return "\n".join(lines)
@@ -126,7 +127,7 @@ class SequenceCache:
             if g.need.kind == "kv":
                 kv = (len(g.entries) * 2 * self.n_pages * g.need.kv_heads * self.page_size * g.need.head_dim
                       * _element_size(self.dtype))
-            else:
+            if g.need.state_shape:
                 count = 1
                 for axis in g.need.state_shape:
                     count *= axis
@@ -145,7 +146,7 @@ class SequenceCache:
                 g.k = torch.zeros((*head, self.page_size, g.need.head_dim), dtype=self.dtype, device=self.device)
                 g.v = torch.zeros((*head, g.need.head_dim, self.page_size), dtype=self.dtype, device=self.device)
                 g.free_pages = list(range(self.n_pages - 1, -1, -1))   # pop() hands out page 0 first
-            else:
+            if g.need.state_shape:
                 g.state = torch.zeros((len(g.entries), self.max_slots, *g.need.state_shape),
                                       dtype=g.need.state_dtype, device=self.device)
         self._allocated = True
@@ -168,7 +169,7 @@ class SequenceCache:
         for g in self.groups:
             if g.need.kind == "kv":
                 g.pages_of[slot] = []
-            elif g.state is not None:
+            if g.state is not None:
                 g.state[:, slot].zero_()
         return slot
 
@@ -231,7 +232,7 @@ class SequenceCache:
         # never read).
         self._state_before = []
         for g in self.groups:
-            if g.need.kind == "state" and g.state is not None:
+            if g.state is not None:
                 index = torch.tensor([slot for slot, _ in requests], dtype=torch.long, device=self.device)
                 self._state_before.append((g, index, g.state.index_select(1, index)))
 
@@ -305,8 +306,8 @@ class SequenceCache:
         g = self.group_of_entry[entry]
         at = g.index_of[entry]
         if g.need.kind == "kv":
-            return LayerCache(g.need, writes, k_pages=g.k[at], v_pages=g.v[at],
-                              page_table=tables[self.groups.index(g)])
+            return LayerCache(g.need, writes, k_pages=g.k[at], v_pages=g.v[at], page_table=tables[self.groups.index(g)],
+                              state=g.state[at] if g.state is not None else None)
         return LayerCache(g.need, writes, state=g.state[at])
 
     # ---- self-check, for tests ----

@@ -3,5 +3,6 @@
 from .base import ConfigError, ConfigReader, LayerKinds, architecture_name, read_config_json
 from .qwen3 import Qwen3Config
 from .gokazen import GokazenConfig
+from .pudorax import PudoraxConfig
 
-__all__ = ["ConfigError", "ConfigReader", "architecture_name", "read_config_json", "LayerKinds", "Qwen3Config", "GokazenConfig"]
+__all__ = ["ConfigError", "ConfigReader", "architecture_name", "read_config_json", "LayerKinds", "Qwen3Config", "GokazenConfig", "PudoraxConfig"]

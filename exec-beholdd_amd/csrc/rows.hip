@@ -1,0 +1,149 @@
+// Small row-wise operations on the float32 residual and on logits:
+//   layernorm        (x - mean) / sqrt(var + eps) * w + b per row, optional row gather, rows or blocks of rows out
+//   cast_concat      [a | b] per row from float32 into the activation type (b optional): the input of a product
+//   softcap          x <- cap * tanh(x / cap) in place
+//   rms_scale_add    h <- h + y / sqrt(mean(y^2) + eps) * w per row
+//   gelu_gate_table  out[r][i] = gelu_tanh(gate[r][i]) * table[token of r][first + i]
+// All statistics are float32.
+#include "common.h"
+
+// One workgroup a row.  The mean first, then the mean of the squared deviations (not E[x^2] - mean^2, which
+// loses digits where the mean is large beside the spread).
+template <typename TO>
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                                                        const float* __restrict__ w, const float* __restrict__ b,
+                                                        TO* __restrict__ out, int width, float eps, int out_block_rows) {
+  __shared__ float scratch[8];
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) sum += src[i];
+  const float mean = block_sum(sum, scratch) / (float)width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float d = src[i] - mean;
+    ss += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float y = (src[i] - mean) * inv * w[i] + (b ? b[i] : 0.f);
+    out[bh_rows_index(out_block_rows, r, i, width)] = from_f32<TO>(y);
+  }
+}
+
+extern "C" int bh_layernorm(const float* x, const int32_t* rows, const float* w, const float* b, void* out, int out_dtype,
+                            int n_rows, int width, float eps, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "layernorm: sizes must be positive");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && width % 32 == 0 && out_dtype == BH_BF16),
+             "layernorm: rows in blocks of %d of width %d are not written", out_block_rows, width);
+  if (out_dtype == BH_F32)
+    layernorm_kernel<float><<<n_rows, 256, 0, stream>>>(x, rows, w, b, (float*)out, width, eps, out_block_rows);
+  else if (out_dtype == BH_BF16)
+    layernorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, rows, w, b, (bf16_t*)out, width, eps, out_block_rows);
+  else
+    return bh_fail("layernorm: unknown dtype %d", out_dtype);
+  return bh_check_launch("layernorm");
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void cast_concat_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                          TO* __restrict__ out, int n_rows, int width, int out_block_rows) {
+  const int total = b ? 2 * width : width;
+  const size_t n = (size_t)n_rows * total;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
+    const int r = (int)(e / total), i = (int)(e % total);
+    const float v = i < width ? a[(size_t)r * width + i] : b[(size_t)r * width + i - width];
+    out[bh_rows_index(out_block_rows, r, i, total)] = from_f32<TO>(v);
+  }
+}
+
+extern "C" int bh_cast_concat(const float* a, const float* b, void* out, int out_dtype, int n_rows, int width,
+                              int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "cast_concat: sizes must be positive");
+  const int total = b ? 2 * width : width;
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && total % 32 == 0 && out_dtype == BH_BF16),
+             "cast_concat: rows in blocks of %d of width %d are not written", out_block_rows, total);
+  const size_t n = (size_t)n_rows * total;
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (out_dtype == BH_F32)
+    cast_concat_kernel<float><<<blocks, 256, 0, stream>>>(a, b, (float*)out, n_rows, width, out_block_rows);
+  else if (out_dtype == BH_BF16)
+    cast_concat_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, b, (bf16_t*)out, n_rows, width, out_block_rows);
+  else
+    return bh_fail("cast_concat: unknown dtype %d", out_dtype);
+  return bh_check_launch("cast_concat");
+}
+
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, long n, float cap) {
+  const float inv = 1.0f / cap;
+  for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long)gridDim.x * blockDim.x)
+    x[e] = cap * tanhf(x[e] * inv);
+}
+
+extern "C" int bh_softcap(float* x, long n, float cap, hipStream_t stream) {
+  BH_REQUIRE(n > 0 && cap > 0.f, "softcap: a positive count and a positive cap");
+  const long blocks = (n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096;
+  softcap_kernel<<<(int)blocks, 256, 0, stream>>>(x, n, cap);
+  return bh_check_launch("softcap");
+}
+
+__global__ __launch_bounds__(256) void rms_scale_add_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                            const float* __restrict__ w, int width, float eps) {
+  __shared__ float scratch[8];
+  const float* src = y + (size_t)blockIdx.x * width;
+  float* dst = h + (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += src[i] * src[i];
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] += src[i] * inv * w[i];
+}
+
+extern "C" int bh_rms_scale_add(float* h, const float* y, const float* w, int n_rows, int width, float eps, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "rms_scale_add: sizes must be positive");
+  rms_scale_add_kernel<<<n_rows, 256, 0, stream>>>(h, y, w, width, eps);
+  return bh_check_launch("rms_scale_add");
+}
+
+__device__ inline float gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// A row's token is tokens[row], or fed[token_src[row]] where token_src is given and not negative (a token chosen on the
+// device that the host has not read yet).
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_gate_table_kernel(const T* __restrict__ gate, const int32_t* __restrict__ tokens,
+                                                              const int32_t* __restrict__ token_src, const int32_t* __restrict__ fed,
+                                                              const T* __restrict__ table, int table_width, int first, int vocab,
+                                                              T* __restrict__ out, int n_rows, int dim, int out_block_rows) {
+  const size_t n = (size_t)n_rows * dim;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
+    const int r = (int)(e / dim), i = (int)(e % dim);
+    int token = tokens[r];
+    if (token_src != nullptr && token_src[r] >= 0) token = fed[token_src[r]];
+    token = token < 0 ? 0 : (token >= vocab ? vocab - 1 : token);
+    const float g = gelu_tanh(to_f32(gate[(size_t)r * dim + i])) * to_f32(table[(size_t)token * table_width + first + i]);
+    out[bh_rows_index(out_block_rows, r, i, dim)] = from_f32<T>(g);
+  }
+}
+
+extern "C" int bh_gelu_gate_table(const void* gate, int dtype, const int32_t* tokens, const int32_t* token_src,
+                                  const int32_t* fed, const void* table, int table_width, int first, int vocab, void* out,
+                                  int n_rows, int dim, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && dim > 0 && vocab > 0, "gelu_gate_table: sizes must be positive");
+  BH_REQUIRE(first >= 0 && first + dim <= table_width, "gelu_gate_table: columns %d..%d lie outside a table row of %d", first,
+             first + dim, table_width);
+  BH_REQUIRE((token_src == nullptr) == (fed == nullptr), "gelu_gate_table: fed tokens come with their source indices");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && dim % 32 == 0 && dtype == BH_BF16),
+             "gelu_gate_table: rows in blocks of %d of width %d are not written", out_block_rows, dim);
+  const size_t n = (size_t)n_rows * dim;
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (dtype == BH_F32)
+    gelu_gate_table_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate, tokens, token_src, fed, (const float*)table,
+                                                            table_width, first, vocab, (float*)out, n_rows, dim, out_block_rows);
+  else if (dtype == BH_BF16)
+    gelu_gate_table_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gate, tokens, token_src, fed, (const bf16_t*)table,
+                                                             table_width, first, vocab, (bf16_t*)out, n_rows, dim, out_block_rows);
+  else
+    return bh_fail("gelu_gate_table: unknown dtype %d", dtype);
+  return bh_check_launch("gelu_gate_table");
+}

@@ -1,0 +1,126 @@
+// What stands around the paged attention kernels for an attention whose queries and keys are normed over the whole
+// projection (all heads of a row together), turned in neighbouring pairs on the first dimensions of each head, and
+// whose heads are gated before the output projection:
+//   whole_norm_rope_write   per row of [q | k | v] (float32): q <- rms(q over all its channels) * wq, k likewise;
+//                           dimensions 2i and 2i+1 (i < turned/2) of every head of q and k turned by
+//                           position * freq[i]; q into a matrix of heads of `pad` dimensions, k and v into the cache
+//                           pages of (sequence, position) as heads of `pad` (zeros beyond dim and vdim), so that keys of
+//                           one size and values of another go through kernels that know one head size
+//   gate_heads              out[row][h][i] = attended[row][h][i] * sigmoid(gate[row][h][i]) for i < vdim
+// Statistics, angles, cosines and sines are float32; the angle is the float32 product position * freq[i].
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_rope_write_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ wq, const float* __restrict__ wk, float eps,
+    const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, const int32_t* __restrict__ page_table,
+    int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write) {
+  __shared__ float scratch[8];
+  const int row = blockIdx.x;
+  const int q_width = H * dim, k_width = G * dim, v_width = G * vdim;
+  const float* q = qkv + (size_t)row * (q_width + k_width + v_width);
+  const float* k = q + q_width;
+  const float* v = k + k_width;
+  const int pos = positions[row];
+  float ss = 0.f;
+  for (int e = threadIdx.x; e < q_width; e += blockDim.x) ss += q[e] * q[e];
+  const float inv_q = 1.0f / sqrtf(block_sum(ss, scratch) / (float)q_width + eps);
+  for (int e = threadIdx.x; e < H * pad; e += blockDim.x) {
+    const int head = e / pad, i = e % pad;
+    float y = 0.f;
+    if (i < dim) {
+      const int at = head * dim + i;
+      y = q[at] * inv_q * wq[at];
+      if (i < turned) {
+        const int mate = at ^ 1;
+        const float other = q[mate] * inv_q * wq[mate];
+        const float angle = (float)pos * freq[i >> 1];
+        const float c = cosf(angle), s = sinf(angle);
+        y = (i & 1) ? y * c + other * s : y * c - other * s;
+      }
+    }
+    q_out[(size_t)row * H * pad + e] = from_f32<T>(y);
+  }
+  if (!write) return;
+  ss = 0.f;
+  for (int e = threadIdx.x; e < k_width; e += blockDim.x) ss += k[e] * k[e];
+  const float inv_k = 1.0f / sqrtf(block_sum(ss, scratch) / (float)k_width + eps);
+  const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE], token = pos % BH_PAGE;
+  for (int e = threadIdx.x; e < G * pad; e += blockDim.x) {
+    const int head = e / pad, i = e % pad;
+    float y = 0.f;
+    if (i < dim) {
+      const int at = head * dim + i;
+      y = k[at] * inv_k * wk[at];
+      if (i < turned) {
+        const int mate = at ^ 1;
+        const float other = k[mate] * inv_k * wk[mate];
+        const float angle = (float)pos * freq[i >> 1];
+        const float c = cosf(angle), s = sinf(angle);
+        y = (i & 1) ? y * c + other * s : y * c - other * s;
+      }
+    }
+    T* keys = k_pages + ((size_t)page * G + head) * BH_PAGE * pad;
+    T* values = v_pages + ((size_t)page * G + head) * BH_PAGE * pad;
+    keys[bh_key_index(kv_order, token, i, pad)] = from_f32<T>(y);
+    values[bh_value_index(kv_order, token, i, pad)] = from_f32<T>(i < vdim ? v[head * vdim + i] : 0.f);
+  }
+}
+
+extern "C" int bh_whole_norm_rope_write(const float* qkv, const float* wq, const float* wk, float eps, const float* freq,
+                                        int turned, const int32_t* positions, const int32_t* row_seq, void* q_out, int dtype,
+                                        void* k_pages, void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
+                                        int H, int G, int dim, int vdim, int pad, int kv_order, int write, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && G > 0 && dim > 0 && vdim > 0, "whole_norm_rope_write: sizes must be positive");
+  BH_REQUIRE(pad >= dim && pad >= vdim, "whole_norm_rope_write: heads of %d do not hold keys of %d and values of %d", pad, dim, vdim);
+  BH_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= dim && dim % 2 == 0 || turned == 0,
+             "whole_norm_rope_write: %d turned dimensions of %d", turned, dim);
+  BH_REQUIRE(turned == 0 || freq != nullptr, "whole_norm_rope_write: a rotation needs its frequencies");
+  BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && pad % 32 == 0),
+             "whole_norm_rope_write: cache order %d does not exist for head size %d", kv_order, pad);
+  if (dtype == BH_F32)
+    whole_norm_rope_write_kernel<float><<<n_rows, 256, 0, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq, (float*)q_out,
+                                                                  (float*)k_pages, (float*)v_pages, page_table, table_stride, H, G,
+                                                                  dim, vdim, pad, kv_order, write);
+  else if (dtype == BH_BF16)
+    whole_norm_rope_write_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq,
+                                                                   (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, page_table,
+                                                                   table_stride, H, G, dim, vdim, pad, kv_order, write);
+  else
+    return bh_fail("whole_norm_rope_write: unknown dtype %d", dtype);
+  return bh_check_launch("whole_norm_rope_write");
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gate_heads_kernel(const T* __restrict__ attended, int pad, const T* __restrict__ gate,
+                                                         int gate_stride, int gate_first, T* __restrict__ out, int n_rows, int H,
+                                                         int vdim, int out_block_rows) {
+  const int width = H * vdim;
+  const size_t n = (size_t)n_rows * width;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
+    const int r = (int)(e / width), c = (int)(e % width), head = c / vdim, i = c % vdim;
+    const float a = to_f32(attended[((size_t)r * H + head) * pad + i]);
+    const float g = to_f32(gate[(size_t)r * gate_stride + gate_first + c]);
+    out[bh_rows_index(out_block_rows, r, c, width)] = from_f32<T>(a / (1.0f + expf(-g)));
+  }
+}
+
+extern "C" int bh_gate_heads(const void* attended, int dtype, int pad, const void* gate, int gate_stride, int gate_first,
+                             void* out, int n_rows, int H, int vdim, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && vdim > 0 && pad >= vdim, "gate_heads: sizes do not fit");
+  BH_REQUIRE(gate_first >= 0 && gate_first + H * vdim <= gate_stride, "gate_heads: the gate lies outside its row");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && (H * vdim) % 32 == 0 && dtype == BH_BF16),
+             "gate_heads: rows in blocks of %d of width %d are not written", out_block_rows, H * vdim);
+  const size_t n = (size_t)n_rows * H * vdim;
+  const int blocks = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  if (dtype == BH_F32)
+    gate_heads_kernel<float><<<blocks, 256, 0, stream>>>((const float*)attended, pad, (const float*)gate, gate_stride, gate_first,
+                                                       (float*)out, n_rows, H, vdim, out_block_rows);
+  else if (dtype == BH_BF16)
+    gate_heads_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)attended, pad, (const bf16_t*)gate, gate_stride, gate_first,
+                                                        (bf16_t*)out, n_rows, H, vdim, out_block_rows);
+  else
+    return bh_fail("gate_heads: unknown dtype %d", dtype);
+  return bh_check_launch("gate_heads");
+}

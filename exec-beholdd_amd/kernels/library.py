@@ -173,6 +173,21 @@ class KernelSizes:
             "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, i, i, i, i, i, p],
             "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, i, p],
             "bh_rotate_heads": [p, ctypes.c_long, i, i, p, ctypes.c_long, i, i, i, p, i, p, i, i, i, p],
+            "bh_layernorm": [p, p, p, p, p, i, i, i, f, i, p],
+            "bh_cast_concat": [p, p, p, i, i, i, i, p],
+            "bh_softcap": [p, ctypes.c_long, f, p],
+            "bh_rms_scale_add": [p, p, p, i, i, f, p],
+            "bh_gelu_gate_table": [p, i, p, p, p, p, i, i, i, p, i, i, i, p],
+            "bh_short_conv": [p, i, i, i, p, p, p, ctypes.c_long, p, p, p, p, i, i, i, i, p],
+            "bh_short_conv_state": [p, i, i, i, p, ctypes.c_long, p, p, i, i, i, p],
+            "bh_whole_norm_rope_write": [p, p, p, f, p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, i, p],
+            "bh_gate_heads": [p, i, i, p, i, i, p, i, i, i, i, p],
+            "bh_ssm_scan": [p, i, p, i, i, i, p, p, p, p, ctypes.c_long, p, p, p, i, i, i, i, i, p],
+            "bh_gated_group_rmsnorm": [p, p, i, i, i, p, f, p, i, i, i, i, p],
+            "bh_route_top_k": [p, p, p, p, i, i, i, p],
+            "bh_experts_gate_up": [p, i, p, p, p, i, i, i, i, f, f, p],
+            "bh_experts_down": [p, i, p, p, p, p, i, i, i, i, p],
+            "bh_clamped_glu": [p, i, p, i, i, f, f, i, p],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
@@ -914,6 +929,210 @@ class HipKernels(KernelSizes):
             self._ptr(x, "rotate_heads x"), x.shape[1], int(x_head), int(x_first), self._ptr(y, "rotate_heads y"), y.shape[1],
             int(y_head), int(y_first), _code(x, "rotate_heads x"), self._ptr(freq, "rotation frequencies", (torch.float32,), True),
             int(turned), self._ptr(positions, "positions", (torch.int32,)), n_rows, n_heads, int(width), self._stream()))
+
+    # ---- row-wise operations on the residual and on logits ----
+    def layernorm(self, x, weight, bias, eps, out, rows=None):
+        """out[r] = (x[row] - mean) / sqrt(var + eps) * weight + bias, row = rows[r] if rows is given else r; x f32 [*, D],
+        weight and bias f32 [D] (bias may be None), out [n, D] in rows or blocks of rows."""
+        n_rows, width = out.shape
+        if x.dim() != 2 or x.shape[1] != width or weight.shape != (width,) or (bias is not None and bias.shape != (width,)):
+            raise KernelError(f"layernorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
+        if (rows is None and x.shape[0] != n_rows) or (rows is not None and rows.shape != (n_rows,)):
+            raise KernelError(f"layernorm: the input rows do not fit {n_rows} output rows")
+        self._check(self.lib.bh_layernorm(
+            self._ptr(x, "layernorm x", (torch.float32,)), self._ptr(rows, "layernorm rows", (torch.int32,), True),
+            self._ptr(weight, "layernorm weight", (torch.float32,)), self._ptr(bias, "layernorm bias", (torch.float32,), True),
+            self._ptr(out, "layernorm out"), _code(out, "layernorm out"), n_rows, width, float(eps), _block_rows(out), self._stream()))
+
+    def cast_concat(self, a, b, out):
+        """out[r] = [a[r] | b[r]] in out's type; a, b f32 [n, D] (b may be None), out [n, 2 D] (or [n, D])."""
+        n_rows, width = a.shape
+        total = 2 * width if b is not None else width
+        if tuple(out.shape) != (n_rows, total) or (b is not None and tuple(b.shape) != (n_rows, width)):
+            raise KernelError(f"cast_concat: shapes a {tuple(a.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_cast_concat(
+            self._ptr(a, "cast_concat a", (torch.float32,)), self._ptr(b, "cast_concat b", (torch.float32,), True),
+            self._ptr(out, "cast_concat out"), _code(out, "cast_concat out"), n_rows, width, _block_rows(out), self._stream()))
+
+    def softcap(self, x, cap):
+        """x <- cap * tanh(x / cap) in place; x f32."""
+        self._check(self.lib.bh_softcap(self._ptr(x, "softcap x", (torch.float32,)), x.numel(), float(cap), self._stream()))
+
+    def rms_scale_add(self, hidden, y, weight, eps):
+        """hidden[r] += y[r] / sqrt(mean(y[r]^2) + eps) * weight; all f32."""
+        n_rows, width = hidden.shape
+        if tuple(y.shape) != (n_rows, width) or weight.shape != (width,):
+            raise KernelError(f"rms_scale_add: shapes hidden {tuple(hidden.shape)}, y {tuple(y.shape)} do not fit")
+        self._check(self.lib.bh_rms_scale_add(
+            self._ptr(hidden, "rms_scale_add hidden", (torch.float32,)), self._ptr(y, "rms_scale_add y", (torch.float32,)),
+            self._ptr(weight, "rms_scale_add weight", (torch.float32,)), n_rows, width, float(eps), self._stream()))
+
+    def gelu_gate_table(self, gate, tokens, table, first, out, token_src=None, fed_tokens=None):
+        """out[r, i] = gelu_tanh(gate[r, i]) * table[token of r, first + i]; gate, out [n, dim], table [V, W] of one type."""
+        n_rows, dim = gate.shape
+        if tuple(out.shape) != (n_rows, dim) or tokens.shape != (n_rows,) or table.dim() != 2 or table.dtype != gate.dtype \
+                or out.dtype != gate.dtype:
+            raise KernelError(f"gelu_gate_table: shapes gate {tuple(gate.shape)}, table {tuple(table.shape)} do not fit")
+        if (token_src is None) != (fed_tokens is None) or (token_src is not None and token_src.shape != (n_rows,)):
+            raise KernelError("gelu_gate_table: fed tokens come with one source index per row")
+        self._check(self.lib.bh_gelu_gate_table(
+            self._ptr(gate, "gelu_gate_table gate"), _code(gate, "gelu_gate_table gate"), self._ptr(tokens, "tokens", (torch.int32,)),
+            self._ptr(token_src, "token_src", (torch.int32,), True), self._ptr(fed_tokens, "fed tokens", (torch.int32,), True),
+            self._ptr(table, "gelu_gate_table table"), table.shape[1], int(first), table.shape[0], self._ptr(out, "gelu_gate_table out"),
+            n_rows, dim, _block_rows(out), self._stream()))
+
+    # ---- a short convolution over time, continued through a state ----
+    @staticmethod
+    def _state_view(state, offset, floats, what):
+        """(address of the region at `offset` floats into every slot's row of `state`, floats from slot to slot)."""
+        if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() < 2:
+            raise KernelError(f"{what}: the state is a contiguous float32 tensor [slots, ...]")
+        per_slot = state.numel() // state.shape[0]
+        if offset < 0 or offset + floats > per_slot:
+            raise KernelError(f"{what}: {floats} floats at {offset} do not lie inside a slot's {per_slot}")
+        return state.data_ptr() + 4 * int(offset), per_slot
+
+    def short_conv(self, u, first, weight, bias, state, state_offset, row_seq, seq_start, seq_slot, out, silu=False):
+        """out[t, c] = sum_j weight[c, j] * u[t - taps + 1 + j, first + c] (+ bias[c]) (then silu) over the rows of each
+        sequence of the step; inputs before the step come from the sequence's state region ([taps - 1, C] f32 at
+        `state_offset` floats into state[slot]).  u [n, W], weight f32 [C, taps], out f32 [n, C]."""
+        n_rows, channels = out.shape
+        taps = weight.shape[1]
+        if u.shape[0] != n_rows or weight.shape[0] != channels or (bias is not None and bias.shape != (channels,)):
+            raise KernelError(f"short_conv: shapes u {tuple(u.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
+        where, stride = None, 0      # one tap reads no earlier row
+        if taps > 1:
+            where, stride = self._state_view(state, state_offset, (taps - 1) * channels, "short_conv")
+            self._ptr(state, "short_conv state", (torch.float32,))
+        self._check(self.lib.bh_short_conv(
+            self._ptr(u, "short_conv u"), _code(u, "short_conv u"), u.shape[1], int(first),
+            self._ptr(weight, "short_conv weight", (torch.float32,)), self._ptr(bias, "short_conv bias", (torch.float32,), True),
+            where, stride, self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(seq_start, "seq_start", (torch.int32,)),
+            self._ptr(seq_slot, "seq_slot", (torch.int32,)), self._ptr(out, "short_conv out", (torch.float32,)), n_rows, channels,
+            taps, int(bool(silu)), self._stream()))
+
+    def short_conv_state(self, u, first, channels, taps, state, state_offset, seq_start, seq_slot):
+        """The state after the step: the last taps - 1 inputs of every sequence (old ones where the step brought fewer)."""
+        n_seqs = seq_slot.shape[0]
+        if seq_start.shape != (n_seqs + 1,):
+            raise KernelError("short_conv_state: seq_start has one entry per sequence and one more")
+        where, stride = self._state_view(state, state_offset, (taps - 1) * channels, "short_conv_state")
+        self._ptr(state, "short_conv state", (torch.float32,))
+        self._check(self.lib.bh_short_conv_state(
+            self._ptr(u, "short_conv_state u"), _code(u, "short_conv_state u"), u.shape[1], int(first), where, stride,
+            self._ptr(seq_start, "seq_start", (torch.int32,)), self._ptr(seq_slot, "seq_slot", (torch.int32,)), n_seqs, int(channels),
+            int(taps), self._stream()))
+
+    # ---- attention with queries and keys normed over the whole projection ----
+    def whole_norm_rope_write(self, qkv, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages, v_pages,
+                              page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+        """qkv f32 [n, H dim + G dim + G vdim] -> q_out [n, H pad] and the cache pages of heads of `pad` (see
+        csrc/whole_norm_attention.hip)."""
+        n_rows = qkv.shape[0]
+        if qkv.shape != (n_rows, (n_heads + n_kv_heads) * dim + n_kv_heads * vdim) or tuple(q_out.shape) != (n_rows, n_heads * pad):
+            raise KernelError(f"whole_norm_rope_write: shapes qkv {tuple(qkv.shape)}, q_out {tuple(q_out.shape)} do not fit")
+        if q_weight.shape != (n_heads * dim,) or k_weight.shape != (n_kv_heads * dim,):
+            raise KernelError("whole_norm_rope_write: one norm weight per query channel and per key channel")
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,):
+            raise KernelError("whole_norm_rope_write: positions and row_seq must have one entry per row")
+        if turned and (freq is None or freq.shape != (turned // 2,)):
+            raise KernelError("whole_norm_rope_write: one frequency per turned pair")
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, pad, q_out.dtype, "whole_norm_rope_write")
+        self._check(self.lib.bh_whole_norm_rope_write(
+            self._ptr(qkv, "qkv", (torch.float32,)), self._ptr(q_weight, "q norm", (torch.float32,)),
+            self._ptr(k_weight, "k norm", (torch.float32,)), float(eps), self._ptr(freq, "frequencies", (torch.float32,), True),
+            int(turned), self._ptr(positions, "positions", (torch.int32,)), self._ptr(row_seq, "row_seq", (torch.int32,)),
+            self._ptr(q_out, "q_out"), _code(q_out, "q_out"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
+            self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
+
+    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim):
+        """out[r, h, i] = attended[r, h, i] * sigmoid(gate[r, gate_first + h vdim + i]), i < vdim; attended [n, H pad]."""
+        n_rows = attended.shape[0]
+        if attended.shape != (n_rows, n_heads * pad) or tuple(out.shape) != (n_rows, n_heads * vdim) or gate.shape[0] != n_rows \
+                or gate.dtype != attended.dtype or out.dtype != attended.dtype:
+            raise KernelError(f"gate_heads: shapes attended {tuple(attended.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_gate_heads(
+            self._ptr(attended, "gate_heads attended"), _code(attended, "gate_heads attended"), int(pad), self._ptr(gate, "gate_heads gate"),
+            gate.shape[1], int(gate_first), self._ptr(out, "gate_heads out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
+
+    # ---- a state-space recurrence with a scalar decay per head ----
+    def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
+                 n_state, n_groups):
+        """Per (sequence, head): S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x with dt = softplus(proj[:, dt_first
+        + head] + dt_bias); xbc f32 [n, H vdim + 2 G N] = [x | B | C], S [H, N, vdim] f32 at `state_offset` floats into
+        state[slot], out f32 [n, H vdim]."""
+        n_rows, n_seqs = xbc.shape[0], seq_slot.shape[0]
+        inner = n_heads * vdim
+        if xbc.shape != (n_rows, inner + 2 * n_groups * n_state) or tuple(out.shape) != (n_rows, inner) or proj.shape[0] != n_rows:
+            raise KernelError(f"ssm_scan: shapes xbc {tuple(xbc.shape)}, out {tuple(out.shape)} do not fit")
+        if seq_start.shape != (n_seqs + 1,) or any(t.shape != (n_heads,) for t in (dt_bias, a_log, d_skip)):
+            raise KernelError("ssm_scan: one dt_bias, A_log and D per head, and seq_start with one entry per sequence and one more")
+        where, stride = self._state_view(state, state_offset, n_heads * n_state * vdim, "ssm_scan")
+        self._ptr(state, "ssm_scan state", (torch.float32,))
+        self._check(self.lib.bh_ssm_scan(
+            self._ptr(xbc, "ssm_scan xbc", (torch.float32,)), xbc.shape[1], self._ptr(proj, "ssm_scan proj"), _code(proj, "ssm_scan proj"),
+            proj.shape[1], int(dt_first), self._ptr(dt_bias, "dt_bias", (torch.float32,)), self._ptr(a_log, "A_log", (torch.float32,)),
+            self._ptr(d_skip, "D", (torch.float32,)), where, stride, self._ptr(seq_start, "seq_start", (torch.int32,)),
+            self._ptr(seq_slot, "seq_slot", (torch.int32,)), self._ptr(out, "ssm_scan out", (torch.float32,)), n_seqs, n_heads, vdim,
+            n_state, n_groups, self._stream()))
+
+    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups):
+        """out = rms_g(y * silu(z[:, z_first : z_first + W])) * weight, the root mean square over each of `groups` equal
+        parts of a row; y f32 [n, W], weight f32 [W], out [n, W] of z's type."""
+        n_rows, width = y.shape
+        if tuple(out.shape) != (n_rows, width) or z.shape[0] != n_rows or weight.shape != (width,) or out.dtype != z.dtype:
+            raise KernelError(f"gated_group_rmsnorm: shapes y {tuple(y.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_gated_group_rmsnorm(
+            self._ptr(y, "gated_group_rmsnorm y", (torch.float32,)), self._ptr(z, "gated_group_rmsnorm z"), _code(z, "gated_group_rmsnorm z"),
+            z.shape[1], int(z_first), self._ptr(weight, "gated_group_rmsnorm weight", (torch.float32,)), float(eps),
+            self._ptr(out, "gated_group_rmsnorm out"), n_rows, width, int(groups), _block_rows(out), self._stream()))
+
+    # ---- routed experts ----
+    def route_top_k(self, logits, bias, chosen, weights):
+        """chosen[r] = the `top` largest of logits[r] + bias (largest first, ties to the lower index), weights[r] = softmax over
+        those alone; logits f32 [n, E], chosen int32 [n, top], weights f32 [n, top]."""
+        n_rows, experts = logits.shape
+        top = chosen.shape[1]
+        if chosen.shape != (n_rows, top) or weights.shape != (n_rows, top) or (bias is not None and bias.shape != (experts,)):
+            raise KernelError(f"route_top_k: shapes logits {tuple(logits.shape)}, chosen {tuple(chosen.shape)} do not fit")
+        self._check(self.lib.bh_route_top_k(
+            self._ptr(logits, "router logits", (torch.float32,)), self._ptr(bias, "router bias", (torch.float32,), True),
+            self._ptr(chosen, "chosen", (torch.int32,)), self._ptr(weights, "route weights", (torch.float32,)), n_rows, experts, top,
+            self._stream()))
+
+    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha):
+        """inner[r * top + j] = act(Wg_e h[r], Wu_e h[r]) for e = chosen[r, j]; w_gate_up [E, 2 ff, K] (gate rows, then up rows)."""
+        n_rows, k = h.shape
+        top = chosen.shape[1]
+        experts, twice, k_w = w_gate_up.shape
+        ff = twice // 2
+        if k_w != k or tuple(inner.shape) != (n_rows * top, ff) or chosen.shape[0] != n_rows or w_gate_up.dtype != h.dtype \
+                or inner.dtype != h.dtype:
+            raise KernelError(f"experts_gate_up: shapes h {tuple(h.shape)}, weights {tuple(w_gate_up.shape)}, inner {tuple(inner.shape)} do not fit")
+        self._check(self.lib.bh_experts_gate_up(
+            self._ptr(h, "experts h"), _code(h, "experts h"), self._ptr(chosen, "chosen", (torch.int32,)), self._ptr(w_gate_up, "expert gate/up"),
+            self._ptr(inner, "experts inner"), n_rows, top, k, ff, float(limit), float(alpha), self._stream()))
+
+    def experts_down(self, inner, chosen, weights, w_down, hidden):
+        """hidden[r] += sum_j weights[r, j] * Wd_e inner[r * top + j], e = chosen[r, j], j in order; w_down [E, D, ff]."""
+        n_rows, top = chosen.shape
+        experts, width, ff = w_down.shape
+        if tuple(inner.shape) != (n_rows * top, ff) or tuple(hidden.shape) != (n_rows, width) or weights.shape != (n_rows, top) \
+                or w_down.dtype != inner.dtype:
+            raise KernelError(f"experts_down: shapes inner {tuple(inner.shape)}, weights {tuple(w_down.shape)}, hidden {tuple(hidden.shape)} do not fit")
+        self._check(self.lib.bh_experts_down(
+            self._ptr(inner, "experts inner"), _code(inner, "experts inner"), self._ptr(chosen, "chosen", (torch.int32,)),
+            self._ptr(weights, "route weights", (torch.float32,)), self._ptr(w_down, "expert down"),
+            self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top, ff, width, self._stream()))
+
+    def clamped_glu(self, gate_up, out, limit, alpha):
+        """out = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit); gate_up [n, 2 ff] = [g | u]."""
+        n_rows, twice = gate_up.shape
+        if tuple(out.shape) != (n_rows, twice // 2) or twice % 2 or out.dtype != gate_up.dtype:
+            raise KernelError(f"clamped_glu: shapes gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_clamped_glu(self._ptr(gate_up, "clamped_glu in"), _code(gate_up, "clamped_glu in"), self._ptr(out, "clamped_glu out"),
+                                            n_rows, twice // 2, float(limit), float(alpha), _block_rows(out), self._stream()))
 
     def stream_read(self, data, workgroups=256, nontemporal=True) -> int:
         """A yardstick, not a product path: read `data` (any contiguous tensor) once the way the streaming kernels

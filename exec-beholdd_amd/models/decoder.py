@@ -15,8 +15,12 @@ from ..parts.embedding import Embedding, LMHead
 
 
 class DecoderModel:
-    def __init__(self, config, embedding, blocks, schedule, final_norm, head, shared_parts=(), residual=None):
+    def __init__(self, config, embedding, blocks, schedule, final_norm, head, shared_parts=(), residual=None,
+                 pass_input=None, pass_starts=()):
         self.config = config
+        # what a pass of a looped stretch is entered through: `pass_input.forward(ctx, hidden, first)` runs ahead of the
+        # scheduled runs `pass_starts`, `first` being what `pass_input.keep` kept of the embedding's output
+        self.pass_input, self.pass_starts = pass_input, frozenset(int(run) for run in pass_starts)
         self.embedding, self.blocks, self.final_norm, self.head = embedding, list(blocks), final_norm, head
         # what turns the embedding's rows into the residual that the blocks update (several streams, say); None: they are it
         self.residual = residual
@@ -52,7 +56,7 @@ class DecoderModel:
         return self.config.max_position
 
     def parts(self):
-        opening = [self.residual] if self.residual is not None else []
+        opening = [part for part in (self.residual, self.pass_input) if part is not None]
         return [self.embedding, *opening, *self.shared_parts, *self.blocks, self.final_norm, self.head]
 
     @property
@@ -61,7 +65,7 @@ class DecoderModel:
         forward depends on the step's device tensors only."""
         return all(getattr(part, "graph_safe", False)
                    for part in (self.embedding, *self.blocks, self.final_norm, self.head)
-                   ) and (self.residual is None or getattr(self.residual, "graph_safe", False))
+                   ) and all(getattr(part, "graph_safe", False) for part in (self.residual, self.pass_input) if part is not None)
 
     @property
     def graph_safe_rows(self) -> int:
@@ -89,8 +93,9 @@ class DecoderModel:
         temporaries are freed before the next one runs; what a block prepares for the next is counted with
         the block that made it), the final norm on the wanted rows and the logits."""
         total = self.embedding.working_bytes(step) if hasattr(self.embedding, "working_bytes") else 0
-        if hasattr(self.residual, "working_bytes"):
-            total += self.residual.working_bytes(step)
+        for part in (self.residual, self.pass_input):
+            if hasattr(part, "working_bytes"):
+                total += part.working_bytes(step)
         widest = max([block.working_bytes(step) for block in self.blocks if hasattr(block, "working_bytes")], default=0)
         last = 0
         if hasattr(self.final_norm, "working_bytes"):
@@ -113,9 +118,15 @@ class DecoderModel:
         hidden = self.embedding.forward(ctx)
         if self.residual is not None:
             hidden = self.residual.open(ctx, hidden)
+        entering = self.pass_input is not None and bool(self.pass_starts)
+        first = self.pass_input.keep(ctx, hidden) if entering else None
         prepared = None      # the next block's first norm, when the block before could prepare it
         for run, (layer, _entry) in enumerate(self.schedule):
+            if entering and run in self.pass_starts:
+                self.pass_input.forward(ctx, hidden, first)
             following = self.blocks[self.schedule[run + 1][0]] if run + 1 < len(self.schedule) else None
+            if entering and run + 1 in self.pass_starts:
+                following = None      # the residual changes between the two blocks: nothing of the next norm can be made ahead
             prepared = self.blocks[layer].forward(ctx, hidden, cache_for_run(run), prepared, following)
         if want_rows is None or want_rows.numel() == 0:
             return None
@@ -128,7 +139,8 @@ class DecoderModel:
 def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.layers.{}.",
                   embedding_name: str = "model.embed_tokens.weight", final_norm_name: str = "model.norm.weight",
                   head_name: str = "lm_head.weight", final_norm_kind: str = "rmsnorm",
-                  make_embedding=None, make_head=None, make_residual=None) -> DecoderModel:
+                  make_embedding=None, make_head=None, make_residual=None, make_shared=None,
+                  make_pass_input=None) -> DecoderModel:
     """Put a decoder together from the registered parts that `config` names.
 
     `position_encoding` is the registered name of the one encoding that all layers share, or a dictionary
@@ -137,8 +149,13 @@ def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.l
     `make_head(config, embedding)` replace the plain embedding and head (a scaled embedding, a head that caps
     its logits); each returns a part with the interface of `parts.embedding`'s.  `make_residual(config)` returns a part
     whose `open(ctx, rows)` turns the embedding's rows into the residual that the blocks update and the final norm
-    reads (several streams: `parts.streams.StreamsResidual`)."""
+    reads (several streams: `parts.streams.StreamsResidual`).  `make_shared(config)` returns {key: part} of parts that the
+    model owns once and the layers' builders find in `shared[key]` (a table that every layer reads a slice of).
+    `make_pass_input(config)` returns the part through which the passes of a looped stretch are entered (or None); the
+    configuration's `pass_starts()` names the scheduled runs it stands ahead of."""
     shared = {}
+    owned = dict(make_shared(config)) if make_shared else {}
+    shared.update(owned)
     labelled = position_encoding if isinstance(position_encoding, dict) else {"default": position_encoding}
     encodings = {label: POSITION_ENCODINGS.get(name)(config, shared) for label, name in labelled.items()}
     shared["position_encodings"] = encodings
@@ -154,5 +171,8 @@ def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.l
         head = LMHead(config.vocab, config.hidden, None, tied_to=embedding)
     else:
         head = LMHead(config.vocab, config.hidden, head_name)
+    pass_input = make_pass_input(config) if make_pass_input else None
     return DecoderModel(config, embedding, blocks, config.schedule(), final_norm, head,
-                        shared_parts=list(encodings.values()), residual=make_residual(config) if make_residual else None)
+                        shared_parts=list(encodings.values()) + list(owned.values()),
+                        residual=make_residual(config) if make_residual else None, pass_input=pass_input,
+                        pass_starts=config.pass_starts() if pass_input is not None else ())

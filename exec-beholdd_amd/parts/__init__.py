@@ -3,7 +3,7 @@
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, LayerCache,
                    Registry, StepContext)
 from .linear import Linear
-from .norm import RMSNorm, ZeroCentredRMSNorm
+from .norm import LayerNorm, RMSNorm, ZeroCentredRMSNorm
 from .rope import NoPositionEncoding, RotaryEncoding, RotaryFrequencies
 from .attention import GQAAttention
 from .mlp import SquaredReLU, SwiGLU
@@ -11,10 +11,15 @@ from .lightning import LightningAttention
 from .latent_attention import LatentAttention
 from .streams import StreamConnection, StreamMixingBlock, StreamsResidual
 from .block import PreNormBlock
-from .embedding import Embedding, LMHead, ScaledLMHead
+from .embedding import CappedLMHead, Embedding, LMHead, ScaledEmbedding, ScaledLMHead
+from .conv_attention import ConvGatedAttention
+from .state_space import StateSpaceScan
+from .experts import ClampedGLU, RoutedExperts
+from .token_side import LoopInput, TokenSideInput, TokenSideTable
 
 __all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "CacheNeed", "LayerCache",
            "Registry", "StepContext", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEncoding",
            "GQAAttention", "SwiGLU", "PreNormBlock", "Embedding", "LMHead", "ZeroCentredRMSNorm", "RotaryFrequencies",
            "SquaredReLU", "LightningAttention", "LatentAttention", "StreamConnection", "StreamMixingBlock", "StreamsResidual",
-           "ScaledLMHead"]
+           "ScaledLMHead", "LayerNorm", "CappedLMHead", "ScaledEmbedding", "ConvGatedAttention", "StateSpaceScan", "ClampedGLU",
+           "RoutedExperts", "LoopInput", "TokenSideInput", "TokenSideTable"]

@@ -78,7 +78,9 @@ class CacheNeed:
     """Storage one layer needs for each sequence.
 
     kind "kv":    keys and values of `kv_heads` heads of `head_dim` for every position, or for
-                  the last `window` positions only (window 0 = all); paged.
+                  the last `window` positions only (window 0 = all); paged.  With a `state_shape` the layer
+                  keeps a fixed-size tensor per sequence beside its pages (the last inputs of a short
+                  convolution ahead of the keys, say), under the rules of kind "state".
     kind "state": one tensor of `state_shape` and `state_dtype` per sequence, of fixed size,
                   zero when a sequence starts.
     Layers whose needs are equal share one storage group.
@@ -205,7 +207,7 @@ class LayerCache:
                 page_size], to be written and read through the kernel library only (it orders the
                 elements of a head inside a page as its attention kernels want them); page_table
                 int32 [n_seqs, width] for the sequences of this step, in batch order.
-    state need: state [max_slots, *state_shape]; index it with ctx.seq_slot.
+    state need: state [max_slots, *state_shape]; index it with ctx.seq_slot.  A kv need with a state shape has both.
     `writes` is False when the schedule lets this layer read another layer's entry.
     """
     need: CacheNeed

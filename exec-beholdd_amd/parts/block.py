@@ -11,12 +11,17 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, graph_rows_allowed
 
 
 class PreNormBlock:
-    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+    """`feed_forward` (with its norm) may be None: a layer of a mixer alone.  `after`: parts that run once the layer's
+    sublayers have, each `forward(ctx, hidden)` on the residual (a second input from the token, say)."""
+
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward, after=()):
         self.mixer_norm, self.mixer = mixer_norm, mixer
         self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+        self.after = [part for part in after if part is not None]
 
     def parts(self):
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        sublayer = [self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else []
+        return [self.mixer_norm, self.mixer, *sublayer, *self.after]
 
     @property
     def graph_safe(self):
@@ -40,8 +45,10 @@ class PreNormBlock:
 
     def working_bytes(self, step) -> int:
         """Everything the four parts allocate, as if nothing were freed before the layer ends."""
-        total = 0
+        total = sum(part.working_bytes(step) for part in self.after if hasattr(part, "working_bytes"))
         for norm, consumer in ((self.mixer_norm, self.mixer), (self.feed_forward_norm, self.feed_forward)):
+            if consumer is None:
+                continue
             if hasattr(norm, "working_bytes"):
                 total += norm.working_bytes(step)
             if hasattr(consumer, "working_bytes"):
@@ -82,6 +89,8 @@ class PreNormBlock:
         `next_block`: the block that runs after this one, whose first norm this block's feed-forward
         may prepare.  Returns that prepared input, or None."""
         x = prepared if prepared is not None else self._normed(ctx, self.mixer_norm, self.mixer, hidden)
+        if self.feed_forward is None or self.after:
+            return self._plain(ctx, x, hidden, cache)
         request = self._joined(self.mixer, self.feed_forward_norm, self.feed_forward)
         if request is not None:
             x = self.mixer.forward(ctx, x, hidden, cache, then_norm=request)
@@ -95,6 +104,32 @@ class PreNormBlock:
             return self.feed_forward.forward(ctx, x, hidden, then_norm=request)
         self.feed_forward.forward(ctx, x, hidden)
         return None
+
+
+    def _plain(self, ctx, x, hidden, cache):
+        """The layer without norms that ride on products across its end: what follows the feed-forward reads the finished
+        residual."""
+        self.mixer.forward(ctx, x, hidden, cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(ctx, self._normed(ctx, self.feed_forward_norm, self.feed_forward, hidden), hidden)
+        for part in self.after:
+            part.forward(ctx, hidden)
+        return None
+
+
+@BLOCKS.register("pre_norm_token_side")
+def _build_pre_norm_token_side(config, layer_index, prefix, kinds, shared):
+    """Tensor names: <prefix>norm1 / norm2 (with the norm's own suffixes), <prefix>side.gate / .proj / .norm where the model
+    has a token side table (`shared["token_side_table"]`)."""
+    from .token_side import TokenSideInput
+
+    norm = NORMS.get(kinds.norm)
+    feed_forward = FEED_FORWARDS.get(kinds.feed_forward)(config, layer_index, prefix, shared)
+    table = shared.get("token_side_table")
+    side = TokenSideInput(config.hidden, table.dim, layer_index, table, config.rms_eps, prefix + "side.") if table is not None else None
+    return PreNormBlock(
+        norm(config, config.hidden, prefix + "norm1", shared), MIXERS.get(kinds.mixer)(config, layer_index, prefix, shared),
+        norm(config, config.hidden, prefix + "norm2", shared) if feed_forward is not None else None, feed_forward, after=[side])
 
 
 @BLOCKS.register("pre_norm")

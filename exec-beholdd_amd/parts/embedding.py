@@ -39,6 +39,20 @@ class Embedding:
         return hidden
 
 
+class ScaledEmbedding(Embedding):
+    """hidden[t] = E[token[t]] * scale, the product made in float32."""
+
+    def __init__(self, vocab: int, width: int, name: str, scale: float):
+        super().__init__(vocab, width, name)
+        self.scale = float(scale)
+
+    def forward(self, ctx):
+        hidden = super().forward(ctx)
+        if self.scale != 1.0:
+            ctx.kernels.scale(hidden, self.scale)
+        return hidden
+
+
 class LMHead:
     graph_safe = True      # forward reads only the step's device tensors
     graph_safe_rows = None # ... whatever the number of tokens a sequence brings
@@ -83,4 +97,20 @@ class ScaledLMHead(LMHead):
         logits = super().forward(ctx, x)
         if self.scale != 1.0:
             ctx.kernels.scale(logits, self.scale)
+        return logits
+
+
+class CappedLMHead(LMHead):
+    """logits = cap * tanh((W x) / cap), on the float32 logits; a cap of 0 leaves them as they are."""
+
+    def __init__(self, vocab: int, width: int, name: str | None, cap: float, tied_to: Embedding | None = None):
+        super().__init__(vocab, width, name, tied_to)
+        if cap < 0.0:
+            raise ValueError(f"a cap on the logits is positive (or 0 for none), got {cap}")
+        self.cap = float(cap)
+
+    def forward(self, ctx, x):
+        logits = super().forward(ctx, x)
+        if self.cap:
+            ctx.kernels.softcap(logits, self.cap)
         return logits

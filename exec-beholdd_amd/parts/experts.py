@@ -1,0 +1,128 @@
+"""Routed experts: a mixture of small gated feed-forward layers of which every token uses a few, and a shared one.
+
+    z = Wr h + br                       router logits, float32 (h in the activation type)
+    chosen = the `top` largest of z;  their weights = softmax over the chosen logits alone
+    expert(h) = Wd (g' * sigmoid(alpha g') * (u' + 1)),  g' = min(Wg h, limit),  u' = clamp(Wu h, -limit, limit)
+    out = sum over chosen of weight * expert(h)  +  shared(h)        (the shared expert has the same form and runs for all)
+
+The experts' matrices are kept stacked: gate and up rows of an expert in one [2 ff, width] block, [experts, ...] in
+all.  A step of few rows reads a chosen expert's rows once per (row, expert) pair (`experts_gate_up`, `experts_down`),
+with no step that depends on the routing on the host, so that decode steps can be captured.  A row's result never
+depends on its batch-mates: its experts' shares are added in the order of its own choice.  The routing is left in
+`ctx.extras["routing"]` ((chosen, weights) of the last layer that ran).  Every size and constant is a constructor
+parameter.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..weights.binder import TensorSpec
+from .base import FEED_FORWARDS
+from .linear import Linear
+
+GATE_SLOPE = 1.702      # alpha of the gate's sigmoid
+
+
+class ClampedGLU:
+    """One gated feed-forward of the form above, for every row: out = Wd act(Wg h, Wu h), added to the residual."""
+    graph_safe = True
+    graph_safe_rows = None
+
+    def __init__(self, hidden: int, ff: int, limit: float, prefix: str, alpha: float = GATE_SLOPE):
+        self.hidden, self.ff, self.limit, self.alpha = int(hidden), int(ff), float(limit), float(alpha)
+        self.gate_up = Linear(hidden, [ff, ff], [prefix + "gate", prefix + "up"])
+        self.down = Linear(ff, hidden, prefix + "down")
+
+    @property
+    def input_reader(self):
+        return self.gate_up.reader()
+
+    def tensor_specs(self):
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, get):
+        self.gate_up.load(get)
+        self.down.load(get)
+
+    def prepare(self, kernels):
+        self.gate_up.prepare(kernels)
+        self.down.prepare(kernels)
+
+    def working_bytes(self, step) -> int:
+        return (self.gate_up.working_bytes(step, step.rows) + step.matrix(step.rows, self.ff, reader=self.down.reader_for_plan(step.act_size))
+                + self.down.working_bytes(step, step.rows, accumulate=True))
+
+    def forward(self, ctx, x, hidden, then_norm=None):
+        both = self.gate_up.forward(ctx, x)
+        inner = ctx.new_activations(both.shape[0], self.ff, reader=self.down.reader())
+        ctx.kernels.clamped_glu(both, inner, self.limit, self.alpha)
+        self.down.forward(ctx, inner, out=hidden, accumulate=True)
+        return None
+
+
+class RoutedExperts:
+    graph_safe = True
+    graph_safe_rows = None
+
+    def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared: ClampedGLU | None = None,
+                 alpha: float = GATE_SLOPE):
+        if not 1 <= top <= n_experts:
+            raise ValueError(f"a row uses 1 to {n_experts} experts, got {top}")
+        self.hidden, self.n_experts, self.top, self.ff = int(hidden), int(n_experts), int(top), int(ff)
+        self.limit, self.alpha, self.prefix, self.shared = float(limit), float(alpha), prefix, shared
+        self.router = Linear(hidden, n_experts, prefix + "router")
+        self.router_bias = self.w_gate_up = self.w_down = None
+
+    def tensor_specs(self):
+        specs = self.router.tensor_specs() + [TensorSpec(self.prefix + "router.b", (self.n_experts,), "linear")]
+        for e in range(self.n_experts):
+            specs += [TensorSpec(f"{self.prefix}e{e}.gate", (self.ff, self.hidden), "linear"),
+                      TensorSpec(f"{self.prefix}e{e}.up", (self.ff, self.hidden), "linear"),
+                      TensorSpec(f"{self.prefix}e{e}.down", (self.hidden, self.ff), "linear")]
+        return specs + (self.shared.tensor_specs() if self.shared is not None else [])
+
+    def load(self, get):
+        self.router.load(get)
+        self.router_bias = get(self.prefix + "router.b").to(torch.float32).contiguous()
+        first = get(f"{self.prefix}e0.gate")
+        self.w_gate_up = torch.empty((self.n_experts, 2 * self.ff, self.hidden), dtype=first.dtype, device=first.device)
+        self.w_down = torch.empty((self.n_experts, self.hidden, self.ff), dtype=first.dtype, device=first.device)
+        for e in range(self.n_experts):
+            self.w_gate_up[e, :self.ff].copy_(first if e == 0 else get(f"{self.prefix}e{e}.gate"))
+            self.w_gate_up[e, self.ff:].copy_(get(f"{self.prefix}e{e}.up"))
+            self.w_down[e].copy_(get(f"{self.prefix}e{e}.down"))
+        if self.shared is not None:
+            self.shared.load(get)
+
+    def prepare(self, kernels):
+        self.router.prepare(kernels)
+        if self.shared is not None:
+            self.shared.prepare(kernels)
+
+    def working_bytes(self, step) -> int:
+        total = self.router.working_bytes(step, step.rows, out_size=4) + 2 * step.matrix(step.rows, self.top, 4)
+        total += step.matrix(step.rows * self.top, self.ff)
+        return total + (self.shared.working_bytes(step) if self.shared is not None else 0)
+
+    def forward(self, ctx, x, hidden, then_norm=None):
+        k = ctx.kernels
+        n = x.shape[0]
+        logits = self.router.forward(ctx, x, out_dtype=torch.float32)
+        chosen = torch.empty((n, self.top), dtype=torch.int32, device=ctx.device)
+        weights = ctx.new_f32(n, self.top)
+        k.route_top_k(logits, self.router_bias, chosen, weights)
+        ctx.extras["routing"] = (chosen, weights)
+        inner = ctx.new_activations(n * self.top, self.ff)
+        k.experts_gate_up(x, chosen, self.w_gate_up, inner, self.limit, self.alpha)
+        k.experts_down(inner, chosen, weights, self.w_down, hidden)
+        if self.shared is not None:
+            self.shared.forward(ctx, x, hidden)
+        return None
+
+
+@FEED_FORWARDS.register("routed_experts")
+def _build_routed_experts(config, layer_index, prefix, shared):
+    sizes = config.layers[layer_index].mlp
+    common = ClampedGLU(config.hidden, sizes.shared.ff, sizes.shared.limit, prefix + "mlp.shared.") if sizes.shared is not None else None
+    return RoutedExperts(config.hidden, sizes.experts, sizes.top, sizes.expert.ff, sizes.expert.limit, prefix + "mlp.", shared=common)

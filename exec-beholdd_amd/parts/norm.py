@@ -80,6 +80,46 @@ class ZeroCentredRMSNorm(RMSNorm):
         raise NotImplementedError("this norm does not ride on the products around it")
 
 
+class LayerNorm:
+    """y = (x - mean) / sqrt(var + eps) * w + b, the variance being the mean of the squared deviations; mean, variance
+    and the result are float32 on the float32 residual, only the output is rounded to the activation type.  The bias
+    is the tensor `name + bias_suffix` (None: no bias).  Weight and bias are kept in float32."""
+    graph_safe = True
+    graph_safe_rows = None
+    serves_reader = True
+
+    def __init__(self, width: int, eps: float, name: str, bias_suffix: str | None = ".b"):
+        if not (eps > 0.0):
+            raise ValueError(f"LayerNorm epsilon must be positive, got {eps}")
+        self.width, self.eps, self.name = int(width), float(eps), name
+        self.bias_name = name + bias_suffix if bias_suffix is not None else None
+        self.weight = self.bias = None
+
+    def tensor_specs(self):
+        specs = [TensorSpec(self.name, (self.width,), "norm")]
+        if self.bias_name is not None:
+            specs.append(TensorSpec(self.bias_name, (self.width,), "linear"))
+        return specs
+
+    def load(self, get):
+        self.weight = get(self.name).to(torch.float32).contiguous()
+        self.bias = get(self.bias_name).to(torch.float32).contiguous() if self.bias_name is not None else None
+
+    def forward(self, ctx, hidden, rows=None, reader=None):
+        n = hidden.shape[0] if rows is None else rows.shape[0]
+        out = ctx.new_activations(n, self.width, reader=reader)
+        ctx.kernels.layernorm(hidden, self.weight, self.bias, self.eps, out, rows=rows)
+        return out
+
+    def working_bytes(self, step, rows: int | None = None, reader=None) -> int:
+        return step.matrix(step.rows if rows is None else rows, self.width, reader=reader)
+
+
+@NORMS.register("layernorm")
+def _build_layernorm(config, width, name, shared):
+    return LayerNorm(width, config.rms_eps, name)
+
+
 @NORMS.register("rmsnorm")
 def _build_rmsnorm(config, width, name, shared):
     return RMSNorm(width, config.rms_eps, name)

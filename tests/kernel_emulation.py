@@ -204,6 +204,170 @@ class TorchKernels:
         y[:, :n_heads * y_head].view(n, n_heads, y_head)[:, :, y_first:y_first + width] = \
             self._turn(xs, freq, turned, positions).to(y.dtype)
 
+    # ---- layer norm, casts, caps, the token's side input ----
+    def layernorm(self, x, weight, bias, eps, out, rows=None):
+        self.calls.append("layernorm")
+        src = (x if rows is None else x[rows.long()]).double()
+        centred = src - src.mean(-1, keepdim=True)
+        y = centred / torch.sqrt((centred ** 2).mean(-1, keepdim=True) + eps) * weight.double()
+        if bias is not None:
+            y = y + bias.double()
+        out.copy_(y.to(out.dtype))
+
+    def cast_concat(self, a, b, out):
+        self.calls.append("cast_concat")
+        out.copy_((a if b is None else torch.cat([a, b], dim=1)).to(out.dtype))
+
+    def softcap(self, x, cap):
+        self.calls.append("softcap")
+        x.copy_(cap * torch.tanh(x / cap))
+
+    def rms_scale_add(self, hidden, y, weight, eps):
+        self.calls.append("rms_scale_add")
+        inv = 1.0 / torch.sqrt((y.double() ** 2).mean(-1, keepdim=True) + eps)
+        hidden.add_((y.double() * inv * weight.double()).float())
+
+    def gelu_gate_table(self, gate, tokens, table, first, out, token_src=None, fed_tokens=None):
+        self.calls.append("gelu_gate_table")
+        z = gate.double()
+        g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        out.copy_((g * table[tokens.long(), first:first + gate.shape[1]].double()).to(out.dtype))
+
+    # ---- a short convolution over time with a state ----
+    @staticmethod
+    def _region(state, offset, floats):
+        return state.reshape(state.shape[0], -1)[:, offset:offset + floats]
+
+    def short_conv(self, u, first, weight, bias, state, state_offset, row_seq, seq_start, seq_slot, out, silu=False):
+        self.calls.append("short_conv")
+        channels, taps = weight.shape
+        for b in range(seq_slot.shape[0]):
+            lo, hi, slot = int(seq_start[b]), int(seq_start[b + 1]), int(seq_slot[b])
+            rows = u[lo:hi, first:first + channels].double()
+            if taps > 1:
+                old = self._region(state, state_offset, (taps - 1) * channels)[slot].reshape(taps - 1, channels).double()
+                rows = torch.cat([old, rows], dim=0)
+            y = sum(rows[j:j + hi - lo] * weight[:, j].double()[None, :] for j in range(taps))
+            if bias is not None:
+                y = y + bias.double()[None, :]
+            if silu:
+                y = y / (1 + torch.exp(-y))
+            out[lo:hi] = y.float()
+
+    def short_conv_state(self, u, first, channels, taps, state, state_offset, seq_start, seq_slot):
+        self.calls.append("short_conv_state")
+        if taps == 1:
+            return
+        region = self._region(state, state_offset, (taps - 1) * channels)
+        for b in range(seq_slot.shape[0]):
+            lo, hi, slot = int(seq_start[b]), int(seq_start[b + 1]), int(seq_slot[b])
+            both = torch.cat([region[slot].reshape(taps - 1, channels), u[lo:hi, first:first + channels].float()], dim=0)
+            region[slot] = both[-(taps - 1):].reshape(-1)
+
+    # ---- attention normed over the whole projection ----
+    def whole_norm_rope_write(self, qkv, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages, v_pages,
+                              page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+        self.calls.append("whole_norm_rope_write")
+        n = qkv.shape[0]
+        q_width, k_width = n_heads * dim, n_kv_heads * dim
+        rms = lambda x, w: (x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * w.double())
+        q = rms(qkv[:, :q_width], q_weight).reshape(n, n_heads, dim)
+        k = rms(qkv[:, q_width:q_width + k_width], k_weight).reshape(n, n_kv_heads, dim)
+        v = qkv[:, q_width + k_width:].reshape(n, n_kv_heads, vdim)
+
+        def turn(x):
+            if not turned:
+                return x
+            angles = (positions.float()[:, None] * freq.float()[None, :]).double()[:, None, :]
+            cos, sin = torch.cos(angles), torch.sin(angles)
+            out = x.clone()
+            a, b = x[..., 0:turned:2], x[..., 1:turned:2]
+            out[..., 0:turned:2] = a * cos - b * sin
+            out[..., 1:turned:2] = b * cos + a * sin
+            return out
+
+        wide = torch.zeros(n, n_heads, pad, dtype=torch.float64)
+        wide[..., :dim] = turn(q)
+        q_out.copy_(wide.reshape(n, n_heads * pad).to(q_out.dtype))
+        if not write_kv:
+            return
+        k = turn(k)
+        for row in range(n):
+            pos, seq = int(positions[row]), int(row_seq[row])
+            page = int(page_table[seq, pos // PAGE])
+            k_pages[page, :, pos % PAGE, :] = 0
+            v_pages[page, :, :, pos % PAGE] = 0
+            k_pages[page, :, pos % PAGE, :dim] = k[row].to(k_pages.dtype)
+            v_pages[page, :, :vdim, pos % PAGE] = v[row].to(v_pages.dtype)
+
+    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim):
+        self.calls.append("gate_heads")
+        n = attended.shape[0]
+        a = attended.float().reshape(n, n_heads, pad)[..., :vdim].reshape(n, n_heads * vdim)
+        out.copy_((a * torch.sigmoid(gate[:, gate_first:gate_first + n_heads * vdim].float())).to(out.dtype))
+
+    # ---- a state-space recurrence ----
+    def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
+                 n_state, n_groups):
+        self.calls.append("ssm_scan")
+        inner, per = n_heads * vdim, n_heads // n_groups
+        region = self._region(state, state_offset, n_heads * n_state * vdim)
+        rate = torch.exp(a_log.double())
+        for b in range(seq_slot.shape[0]):
+            lo, hi, slot = int(seq_start[b]), int(seq_start[b + 1]), int(seq_slot[b])
+            s = region[slot].reshape(n_heads, n_state, vdim).double()
+            for row in range(lo, hi):
+                x = xbc[row, :inner].double().reshape(n_heads, vdim)
+                bm = xbc[row, inner:inner + n_groups * n_state].double().reshape(n_groups, n_state).repeat_interleave(per, dim=0)
+                cm = xbc[row, inner + n_groups * n_state:].double().reshape(n_groups, n_state).repeat_interleave(per, dim=0)
+                dt = torch.nn.functional.softplus(proj[row, dt_first:dt_first + n_heads].double() + dt_bias.double(), threshold=40.0)
+                s = (torch.exp(-rate * dt)[:, None, None] * s + (dt[:, None] * bm)[:, :, None] * x[:, None, :]).float().double()
+                out[row] = (torch.einsum("hnv,hn->hv", s, cm) + d_skip.double()[:, None] * x).float().reshape(-1)
+            region[slot] = s.float().reshape(-1)
+
+    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups):
+        self.calls.append("gated_group_rmsnorm")
+        n, width = y.shape
+        g = z[:, z_first:z_first + width].double()
+        v = (y.double() * (g / (1 + torch.exp(-g)))).reshape(n, groups, width // groups)
+        v = (v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps)).reshape(n, width)
+        out.copy_((v * weight.double()).to(out.dtype))
+
+    # ---- routed experts ----
+    @staticmethod
+    def _clamped_glu(g, u, limit, alpha):
+        g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+        return g * torch.sigmoid(alpha * g) * (u + 1.0)
+
+    def route_top_k(self, logits, bias, chosen, weights):
+        self.calls.append("route_top_k")
+        z = logits.double() + (bias.double() if bias is not None else 0.0)
+        order = torch.argsort(-z, dim=-1, stable=True)[:, :chosen.shape[1]]
+        chosen.copy_(order.to(torch.int32))
+        weights.copy_(torch.softmax(torch.gather(z, 1, order), dim=-1).float())
+
+    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha):
+        self.calls.append("experts_gate_up")
+        top, ff = chosen.shape[1], w_gate_up.shape[1] // 2
+        for row in range(h.shape[0]):
+            for j in range(top):
+                both = w_gate_up[int(chosen[row, j])].double() @ h[row].double()
+                inner[row * top + j] = self._clamped_glu(both[:ff], both[ff:], limit, alpha).to(inner.dtype)
+
+    def experts_down(self, inner, chosen, weights, w_down, hidden):
+        self.calls.append("experts_down")
+        top = chosen.shape[1]
+        for row in range(hidden.shape[0]):
+            total = torch.zeros(hidden.shape[1], dtype=torch.float64)
+            for j in range(top):
+                total += float(weights[row, j]) * (w_down[int(chosen[row, j])].double() @ inner[row * top + j].double())
+            hidden[row] += total.float()
+
+    def clamped_glu(self, gate_up, out, limit, alpha):
+        self.calls.append("clamped_glu")
+        ff = out.shape[1]
+        out.copy_(self._clamped_glu(gate_up[:, :ff].double(), gate_up[:, ff:].double(), limit, alpha).to(out.dtype))
+
     def gemm_swiglu(self, a, w, out):
         self.calls.append("gemm_swiglu")
         both = torch.empty(a.shape[0], w.shape[0], dtype=a.dtype)
