@@ -228,7 +228,7 @@ def forward(config, w, tokens, residual_after_runs=None):
     """Logits [T, vocab] of one whole sequence from position 0; `residual_after_runs` collects X after every layer run."""
     eps = config["norm"]["eps"]
     tokens = np.asarray(tokens)
-    x = (w["embed"][tokens].astype(np.float64) * config["embedding"]["scale"]).astype(F32)
+    x = (w["embed"][tokens].astype(np.float64) * (config.get("embedding") or {}).get("scale", 1.0)).astype(F32)
     x0 = x.copy()
     order, firsts = run_order(config)
     side = config.get("token_side")
@@ -257,3 +257,13 @@ def forward(config, w, tokens, residual_after_runs=None):
     if cap:
         logits = cap * np.tanh(logits / cap)
     return logits.astype(F32)
+
+
+def greedy(config, w, prompt, n_new):
+    """The tokens that greedy decoding adds to `prompt` (the whole sequence run again for every token; ties to the lower id)."""
+    fed, out = list(prompt), []
+    for _ in range(n_new):
+        token = int(np.argmax(forward(config, w, fed)[-1]))
+        out.append(token)
+        fed.append(token)
+    return out
