@@ -58,6 +58,11 @@ def parse():
                              "streams) at layer sizes of real models beside Qwen3 at equal width and depth: prefill and decode "
                              "tokens per second of both, and every kernel of the new design beside its like with the fraction "
                              "of its roofline; prints one JSON line and exits")
+    parser.add_argument("--pudorax", action="store_true",
+                        help="the Pudorax design (attention behind short convolutions with a gate, a state-space mixer, routed "
+                             "experts, a per-layer token input, a looped stretch) at layer sizes of real models beside Qwen3 at "
+                             "equal width and as many layer runs: prefill and decode tokens per second of both, and every kernel "
+                             "of the new design beside its like with the fraction of its roofline; prints one JSON line and exits")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
                              "top-k, with top-p on rows of three spreads, with both), print the microseconds and exit")
@@ -395,6 +400,227 @@ def gokazen_bench(args, torch):
     return 0
 
 
+def pudorax_config(width, heads, vocab, experts=32, top=4, expert_ff=None, shared_ff=None, side=256):
+    """Six layers of which two run twice (eight layer runs): attention with heads of 128, four query heads to a key/value
+    head, convolutions of four taps and a rotation over half a head; state-space layers of twice the width in heads of 64
+    with a state of 128 rows; `experts` experts of which `top` are used, and a shared one; a token side input of `side`."""
+    expert_ff, shared_ff = expert_ff or 3 * width // 8, shared_ff or 3 * width // 2
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff, "limit": 7.0},
+           "shared": {"ff": shared_ff, "limit": 7.0}}
+    attention = {"type": "attention", "mlp": mlp,
+                 "mixer": {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+                           "rot": {"base": 1000000.0, "dims": 64}}}
+    mamba = {"type": "mamba2", "mlp": mlp,
+             "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8, "conv": 4}}
+    return {"architecture": "Pudorax", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "norm": {"eps": 1e-6}, "token_side": {"dim": side}, "loop": {"start": 1, "stop": 3, "times": 2},
+            "layers": [attention, mamba, attention, attention, mamba, attention]}
+
+
+def pudorax_kernels(K, torch, width, heads, context, experts=32, top=4):
+    """Every kernel of the design and its like among the other models', alone, at a prompt of 2,048 rows and at a decode step
+    of 8 rows over `context` cached tokens: microseconds and the fraction of the roofline (the slower of its bytes at the HBM
+    peak and its operations at the peak of the units it runs on)."""
+    from types import SimpleNamespace
+    bf16, f32, dev = torch.bfloat16, torch.float32, "cuda:0"
+    dim = vdim = 128
+    page = K.page_size
+    out = {}
+
+    def note(name, us, n_bytes, flops=0.0, peak=PEAK_FLOPS["fp32"]):
+        floor = max(n_bytes / (PEAK_HBM_GBS * 1e9), flops / peak) * 1e6
+        out[name] = {"us": round(us, 1), "roofline_us": round(floor, 2), "fraction": round(floor / us, 3)}
+
+    def pages_for(n_seqs, length, kv_heads, head):
+        per = -(-length // page)
+        k_pages = torch.randn(n_seqs * per, kv_heads, page, head, device=dev).to(bf16)
+        v_pages = torch.randn(n_seqs * per, kv_heads, head, page, device=dev).to(bf16)
+        table = torch.arange(n_seqs * per, dtype=torch.int32, device=dev).view(n_seqs, per).contiguous()
+        return k_pages, v_pages, table
+
+    kv_heads = max(heads // 4, 1)
+    ones = torch.ones(width, device=dev)
+    for rows, seqs, past, tag in ((2048, 1, 0, "prompt of 2,048"), (8, 8, context - 1, f"decode of 8 at {context}")):
+        each = rows // seqs
+        starts = torch.arange(0, rows + 1, each, dtype=torch.int32, device=dev)
+        slots = torch.arange(seqs, dtype=torch.int32, device=dev)
+        positions = (torch.arange(rows, dtype=torch.int32, device=dev) % each + past).contiguous()
+        row_seq = (torch.arange(rows, dtype=torch.int32, device=dev) // each).contiguous()
+        layout = SimpleNamespace(seq_start=starts, n_seqs=seqs, max_rows_per_seq=each, max_position=past + each - 1)
+        hidden = torch.randn(rows, width, device=dev)
+        normed = torch.empty(rows, width, device=dev, dtype=bf16)
+        # -- norms
+        us = timed(lambda: K.layernorm(hidden, ones, ones, 1e-6, normed), torch)
+        note(f"layernorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        us = timed(lambda: K.rmsnorm(hidden, ones, 1e-6, normed), torch)
+        note(f"qwen3 rmsnorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        # -- attention: convolution, norm over the projection, rotation and cache write; the gate
+        q_w, k_w = heads * dim, kv_heads * dim
+        conv_w = q_w + 2 * k_w
+        proj = torch.randn(rows, conv_w + q_w, device=dev).to(bf16)
+        taps = 4
+        conv_weight = torch.randn(conv_w, taps, device=dev)
+        conv_state = torch.zeros(seqs, (taps - 1) * conv_w, device=dev)
+        conv = torch.empty(rows, conv_w, device=dev)
+        k_pages, v_pages, table = pages_for(seqs, past + each, kv_heads, dim)
+        q_out = torch.empty(rows, heads * dim, device=dev, dtype=bf16)
+        freq = torch.ones(32, device=dev)
+        wq, wk = torch.ones(q_w, device=dev), torch.ones(k_w, device=dev)
+
+        def convolved_write():
+            K.short_conv(proj, 0, conv_weight, None, conv_state, 0, row_seq, starts, slots, conv)
+            K.short_conv_state(proj, 0, conv_w, taps, conv_state, 0, starts, slots)
+            K.whole_norm_rope_write(conv, wq, wk, 1e-6, freq, 64, positions, row_seq, q_out, k_pages, v_pages, table, heads, kv_heads,
+                                    dim, vdim, dim, True)
+        us = timed(convolved_write, torch)
+        note(f"short_conv + state + whole_norm_rope_write, {tag}", us, 2 * rows * conv_w * 2)
+        head_weight = torch.ones(dim, device=dev)
+        cos = torch.ones(past + each, dim // 2, device=dev)
+        qkv = torch.randn(rows, conv_w, device=dev).to(bf16)
+        us = timed(lambda: K.qk_norm_rope_cache(qkv, q_out, head_weight, head_weight, 1e-6, cos, cos, positions, row_seq, k_pages, v_pages,
+                                                table, heads, kv_heads, dim, True, past + each - 1), torch)
+        note(f"qwen3 qk_norm_rope_cache, {tag}", us, 2 * qkv.numel() * 2)
+        attended = torch.empty_like(q_out)
+        us = timed(lambda: K.attention(q_out, attended, k_pages, v_pages, table, row_seq, positions, heads, kv_heads, dim, dim ** -0.5, 0, layout=layout), torch)
+        keys_seen = seqs * (past + each) if each == 1 else each * (each + 1) // 2
+        note(f"attention ({heads} heads on {kv_heads} of {dim}; the framework's own), {tag}", us,
+             2 * seqs * (past + each) * kv_heads * dim * 2 + 2 * q_out.numel() * 2, 4.0 * keys_seen * heads * dim, PEAK_FLOPS["bf16"])
+        gated = torch.empty(rows, q_w, device=dev, dtype=bf16)
+        us = timed(lambda: K.gate_heads(attended, dim, proj, conv_w, gated, heads, vdim), torch)
+        note(f"gate_heads, {tag}", us, 3 * gated.numel() * 2)
+        # -- the state-space mixer
+        s_heads, s_vdim, n_state, groups = 2 * width // 64, 64, 128, 8
+        inner, bc = s_heads * s_vdim, 2 * groups * n_state
+        s_proj = torch.randn(rows, 2 * inner + bc + s_heads, device=dev).to(bf16)
+        s_state = torch.zeros(seqs, s_heads * n_state * s_vdim + (taps - 1) * (inner + bc), device=dev)
+        xbc = torch.empty(rows, inner + bc, device=dev)
+        s_conv_w, s_conv_b = torch.randn(inner + bc, taps, device=dev), torch.zeros(inner + bc, device=dev)
+
+        def s_convolved():
+            K.short_conv(s_proj, inner, s_conv_w, s_conv_b, s_state, s_heads * n_state * s_vdim, row_seq, starts, slots, xbc, silu=True)
+            K.short_conv_state(s_proj, inner, inner + bc, taps, s_state, s_heads * n_state * s_vdim, starts, slots)
+        us = timed(s_convolved, torch)
+        note(f"short_conv with silu + state, {tag}", us, rows * (inner + bc) * (2 + 4))
+        per_head = torch.zeros(s_heads, device=dev)
+        y = torch.empty(rows, inner, device=dev)
+        us = timed(lambda: K.ssm_scan(xbc, s_proj, 2 * inner + bc, per_head, per_head, per_head, s_state, 0, starts, slots, y, s_heads,
+                                      s_vdim, n_state, groups), torch)
+        note(f"ssm_scan, {tag}", us, 2 * seqs * s_heads * n_state * s_vdim * 4 + xbc.numel() * 4 + y.numel() * 4, 6.0 * rows * s_heads * n_state * s_vdim)
+        l_heads = width // 128
+        l_proj = torch.randn(rows, 4 * l_heads * 128, device=dev).to(bf16)
+        l_state = torch.zeros(seqs, l_heads, 128, 128, device=dev)
+        decay = torch.full((l_heads,), 0.99, device=dev)
+        mixed = torch.empty(rows, l_heads * 128, device=dev)
+        us = timed(lambda: K.lightning_scan(l_proj, 0, l_heads * 128, 2 * l_heads * 128, l_state, decay, starts, slots, mixed, l_heads, 128, 128), torch)
+        note(f"gokazen lightning_scan, {tag}", us, 2 * l_state.numel() * 4 + rows * 3 * l_heads * 128 * 2 + mixed.numel() * 4, 4.0 * rows * l_heads * 128 * 128)
+        s_normed = torch.empty(rows, inner, device=dev, dtype=bf16)
+        s_weight = torch.ones(inner, device=dev)
+        us = timed(lambda: K.gated_group_rmsnorm(y, s_proj, 0, s_weight, 1e-6, s_normed, groups), torch)
+        note(f"gated_group_rmsnorm, {tag}", us, y.numel() * 4 + 2 * s_normed.numel() * 2)
+        l_gated = torch.empty(rows, l_heads * 128, device=dev, dtype=bf16)
+        l_weight = torch.ones(l_heads * 128, device=dev)
+        us = timed(lambda: K.gated_rmsnorm(mixed, l_proj, 3 * l_heads * 128, l_weight, 1e-6, l_gated), torch)
+        note(f"gokazen gated_rmsnorm, {tag}", us, mixed.numel() * 4 + 2 * l_gated.numel() * 2)
+        # -- routed experts
+        ff = 3 * width // 8
+        logits = torch.randn(rows, experts, device=dev)
+        chosen = torch.empty(rows, top, dtype=torch.int32, device=dev)
+        shares = torch.empty(rows, top, device=dev)
+        bias = torch.zeros(experts, device=dev)
+        us = timed(lambda: K.route_top_k(logits, bias, chosen, shares), torch)
+        note(f"route_top_k, {tag}", us, logits.numel() * 4 + 2 * chosen.numel() * 4)
+        x = torch.randn(rows, width, device=dev).to(bf16)
+        w_gu = (torch.randn(experts, 2 * ff, width, device=dev) * 0.02).to(bf16)
+        w_d = (torch.randn(experts, width, ff, device=dev) * 0.02).to(bf16)
+        active = int(torch.unique(chosen).numel())
+        for name, call, n_bytes, flops in pudorax_expert_calls(K, torch, x, chosen, shares, w_gu, w_d, hidden, active, top, ff, width):
+            us = timed(call, torch, repeats=5 if rows > 64 else 20)
+            note(f"{name}, {tag}", us, n_bytes, flops, PEAK_FLOPS["bf16"])
+        both = torch.randn(rows, 2 * ff * 4, device=dev).to(bf16)
+        activated = torch.empty(rows, ff * 4, device=dev, dtype=bf16)
+        us = timed(lambda: K.clamped_glu(both, activated, 7.0, 1.702), torch)
+        note(f"clamped_glu, {tag}", us, 3 * activated.numel() * 2)
+        us = timed(lambda: K.swiglu(both, activated), torch)
+        note(f"qwen3 swiglu, {tag}", us, 3 * activated.numel() * 2)
+        # -- the token's side input and the loop's entry
+        side = 256
+        table_w = torch.randn(4096, 6 * side, device=dev).to(bf16)
+        gate = torch.randn(rows, side, device=dev).to(bf16)
+        g_out = torch.empty_like(gate)
+        tokens = torch.randint(0, 4096, (rows,), dtype=torch.int32, device=dev)
+        us = timed(lambda: K.gelu_gate_table(gate, tokens, table_w, 2 * side, g_out), torch)
+        note(f"gelu_gate_table, {tag}", us, 3 * gate.numel() * 2)
+        yy = torch.randn(rows, width, device=dev)
+        us = timed(lambda: K.rms_scale_add(hidden, yy, ones, 1e-6), torch)
+        note(f"rms_scale_add, {tag}", us, 3 * hidden.numel() * 4)
+        wide = torch.empty(rows, 2 * width, device=dev, dtype=bf16)
+        us = timed(lambda: K.cast_concat(hidden, yy, wide), torch)
+        note(f"cast_concat, {tag}", us, 2 * hidden.numel() * 4 + wide.numel() * 2)
+    return out
+
+
+def pudorax_expert_calls(K, torch, x, chosen, shares, w_gu, w_d, hidden, active, top, ff, width):
+    """(name, call, bytes, operations) of the routed experts' work as a step of these rows runs it: grouped by expert, then for
+    few rows a workgroup per expert and block of outputs, for many rows the framework's products on every expert's stretch."""
+    from types import SimpleNamespace
+    from beholdd.parts.experts import RoutedExperts
+    rows, experts = x.shape[0], w_gu.shape[0]
+    pairs = rows * top
+    lists = torch.empty(experts, rows, dtype=torch.int32, device=x.device)
+    counts = torch.empty(experts, dtype=torch.int32, device=x.device)
+    K.experts_group(chosen, lists, counts)
+    weights_read = active * 3 * ff * width * 2
+    yield ("experts_group", lambda: K.experts_group(chosen, lists, counts), pairs * 4 * 2, 0.0)
+    if pairs < RoutedExperts.PRODUCT_PAIRS * experts:
+        inner = torch.empty(pairs, ff, device=x.device, dtype=x.dtype)
+        y = torch.empty(pairs, width, device=x.device)
+        yield ("experts_rows (gate and up)", lambda: K.experts_rows(x, top, lists, counts, w_gu, inner, gated=True, limit=7.0, alpha=1.702),
+               weights_read * 2 // 3 + x.numel() * 2 + inner.numel() * 2, 4.0 * pairs * ff * width)
+        yield ("experts_rows (down)", lambda: K.experts_rows(inner, 1, lists, counts, w_d, y), weights_read // 3 + inner.numel() * 2 + y.numel() * 4,
+               2.0 * pairs * ff * width)
+        yield ("experts_combine", lambda: K.experts_combine(y, None, shares, hidden), y.numel() * 4 + 2 * hidden.numel() * 4, 0.0)
+        return
+    part = RoutedExperts(width, experts, top, ff, 7.0, "m.")
+    part.w_gate_up, part.w_down = w_gu, w_d
+    part.for_products = [(K.pack_weight(w_gu[e]), K.pack_weight(w_d[e])) for e in range(experts)]
+    ctx = SimpleNamespace(kernels=K, device=x.device, new_f32=lambda *shape: torch.empty(shape, device=x.device),
+                          new_activations=lambda *shape, reader=None: torch.empty(shape, device=x.device, dtype=x.dtype))
+    yield (f"experts as products (gather, {2 * experts} products, clamped_glu, combine)", lambda: part._as_products(ctx, x, lists, counts, shares, hidden),
+           weights_read + pairs * (2 * width + 3 * ff) * 2 + pairs * width * 8, 6.0 * pairs * ff * width)
+
+
+def pudorax_bench(args, torch):
+    from beholdd.engine import Engine, random_model_on_device
+
+    device, points = "cuda:0", []
+    t = min(args.prefill_tokens, args.context)
+    for width, heads in ((2048, 16), (4096, 32)):
+        pair = {"pudorax": pudorax_config(width, heads, 32768),
+                "qwen3": dict(QWEN3_8B, num_hidden_layers=8, hidden_size=width, num_attention_heads=heads,
+                              num_key_value_heads=heads // 4, intermediate_size=3 * width, vocab_size=32768)}
+        point = {"width": width, "heads": heads, "layer_runs": 8}
+        for name, config in pair.items():
+            model = random_model_on_device(config, seed=0, dtype="bfloat16", device=device)
+            engine = Engine(model=model, dtype="bfloat16", max_tokens=args.batch * (-(-args.context // 64) * 64),
+                            max_slots=args.batch, device=device)
+            parameters = sum(int(np_prod(spec.shape)) for spec in model.tensor_specs())
+            seconds, _ = decode_run(engine, args.batch, args.context, args.steps, args.warmup, torch)
+            prefill = prefill_run(engine, t, torch)
+            point[name] = {"parameters": parameters, "decode_ms_per_step": round(seconds * 1e3, 4),
+                           "decode_tok_per_s": round(args.batch / seconds, 1), "prefill_ms": round(prefill * 1e3, 3),
+                           "prefill_tok_per_s": round(t / prefill, 1)}
+            kernels = engine.kernels
+            del engine, model
+            torch.cuda.empty_cache()
+        points.append(point)
+    line = {"metric": f"Pudorax beside Qwen3 at equal width and as many layer runs: decode tok/s @ batch {args.batch}, context {args.context}; prefill of {t} tokens",
+            "unit": "tok/s", "value": points[-1]["pudorax"]["decode_tok_per_s"], "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "points": points,
+            "kernels": pudorax_kernels(kernels, torch, 4096, 32, args.context)}
+    print(json.dumps(line))
+    return 0
+
+
 def np_prod(shape):
     total = 1
     for axis in shape:
@@ -416,6 +642,8 @@ def main():
         return 0
     if args.gokazen:
         return gokazen_bench(args, torch)
+    if args.pudorax:
+        return pudorax_bench(args, torch)
 
     from beholdd.engine import Engine, random_model_on_device
 

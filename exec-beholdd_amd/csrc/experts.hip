@@ -15,49 +15,65 @@ __device__ inline float clamped_glu(float g, float u, float limit, float alpha) 
 }
 
 #define ROUTE_MAX_TOP 32
+#define ROUTE_PER_LANE 16      // experts a lane holds: up to 1024 experts
 
-// One thread a row.
-__global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
-                                                        int32_t* __restrict__ chosen, float* __restrict__ weights, int n_rows,
-                                                        int E, int top) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+// One wave a row: a lane holds the logits of experts lane, lane + 64, ...; the largest is found `top` times over, each time
+// without those already taken (ties go to the lower index).
+__global__ __launch_bounds__(256) void route_top_k_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                         int32_t* __restrict__ chosen, float* __restrict__ weights, int n_rows,
+                                                         int E, int top) {
+  const int lane = threadIdx.x & (BH_WAVE - 1), row = blockIdx.x * (blockDim.x / BH_WAVE) + threadIdx.x / BH_WAVE;
   if (row >= n_rows) return;
   const float* z = logits + (size_t)row * E;
-  int picked[ROUTE_MAX_TOP];
-  float value[ROUTE_MAX_TOP];
+  float v[ROUTE_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+    const int e = lane + i * BH_WAVE;
+    v[i] = e < E ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
+  }
+  unsigned taken = 0;      // bit i: this lane's expert lane + 64 i was chosen
+  float largest = 0.f, sum = 0.f, mine = 0.f;      // lane j keeps the j-th choice's exponential
+  int mine_index = 0;
   for (int j = 0; j < top; ++j) {
-    int best = -1;
-    float best_v = 0.f;
-    for (int e = 0; e < E; ++e) {
-      bool taken = false;
-      for (int i = 0; i < j; ++i) taken |= picked[i] == e;
-      if (taken) continue;
-      const float v = z[e] + (bias ? bias[e] : 0.f);
-      if (best < 0 || v > best_v) {
-        best = e;
-        best_v = v;
+    float best = -INFINITY;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+      const int e = lane + i * BH_WAVE;
+      if (e < E && !((taken >> i) & 1u) && (v[i] > best || best_e == 0x7fffffff)) {
+        best = v[i];
+        best_e = e;
       }
     }
-    picked[j] = best;
-    value[j] = best_v;
+#pragma unroll
+    for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, BH_WAVE);
+      const int other_e = __shfl_xor(best_e, off, BH_WAVE);
+      if (other_e != 0x7fffffff && (best_e == 0x7fffffff || other > best || (other == best && other_e < best_e))) {
+        best = other;
+        best_e = other_e;
+      }
+    }
+    if ((best_e & (BH_WAVE - 1)) == lane) taken |= 1u << (best_e / BH_WAVE);
+    if (j == 0) largest = best;
+    const float p = expf(best - largest);
+    sum += p;
+    if (lane == j) {
+      mine = p;
+      mine_index = best_e;
+    }
   }
-  float sum = 0.f;
-  const float largest = value[0];
-  for (int j = 0; j < top; ++j) {
-    value[j] = expf(value[j] - largest);
-    sum += value[j];
-  }
-  for (int j = 0; j < top; ++j) {
-    chosen[(size_t)row * top + j] = picked[j];
-    weights[(size_t)row * top + j] = value[j] / sum;
+  if (lane < top) {
+    chosen[(size_t)row * top + lane] = mine_index;
+    weights[(size_t)row * top + lane] = mine / sum;
   }
 }
 
 extern "C" int bh_route_top_k(const float* logits, const float* bias, int32_t* chosen, float* weights, int n_rows, int E, int top,
                               hipStream_t stream) {
-  BH_REQUIRE(n_rows > 0 && E > 0, "route_top_k: sizes must be positive");
+  BH_REQUIRE(n_rows > 0 && E > 0 && E <= BH_WAVE * ROUTE_PER_LANE, "route_top_k: 1 to %d experts, got %d", BH_WAVE * ROUTE_PER_LANE, E);
   BH_REQUIRE(top >= 1 && top <= E && top <= ROUTE_MAX_TOP, "route_top_k: 1 to min(%d, %d) experts a row, got %d", E, ROUTE_MAX_TOP, top);
-  route_top_k_kernel<<<(n_rows + 63) / 64, 64, 0, stream>>>(logits, bias, chosen, weights, n_rows, E, top);
+  route_top_k_kernel<<<(n_rows + 3) / 4, 256, 0, stream>>>(logits, bias, chosen, weights, n_rows, E, top);
   return bh_check_launch("route_top_k");
 }
 
@@ -181,4 +197,202 @@ extern "C" int bh_clamped_glu(const void* gu, int dtype, void* out, int n_rows, 
   else
     return bh_fail("clamped_glu: unknown dtype %d", dtype);
   return bh_check_launch("clamped_glu");
+}
+
+// ---- the experts' work grouped by expert ----------------------------------------------------------------------
+//   experts_group     for every expert the (row, choice) pairs that chose it, in the pairs' order, and their count
+//   experts_rows      per expert, for its pairs: a product with that expert's matrix, the matrix read from memory once per
+//                     workgroup whatever the number of pairs (gated: two rows an output and the activation; plain: float32
+//                     results for experts_combine)
+//   experts_gather    the pairs' input rows side by side, expert after expert, for products of many rows
+//   experts_combine   h_res[row] += sum_j weight_j * y[place of pair (row, j)], j in order
+
+// One workgroup an expert: it walks over all pairs in order and keeps those that chose it.
+__global__ __launch_bounds__(256) void experts_group_kernel(const int32_t* __restrict__ chosen, int n_pairs, int32_t* __restrict__ list,
+                                                            int capacity, int32_t* __restrict__ counts) {
+  __shared__ int wave_count[4];
+  const int e = blockIdx.x, lane = threadIdx.x & (BH_WAVE - 1), wave = threadIdx.x / BH_WAVE;
+  int base = 0;
+  for (int p0 = 0; p0 < n_pairs; p0 += 256) {
+    const int p = p0 + threadIdx.x;
+    const bool mine = p < n_pairs && chosen[p] == e;
+    const unsigned long long mask = __ballot(mine);
+    const int before = __popcll(mask & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[wave] = __popcll(mask);
+    __syncthreads();
+    int offset = base, total = 0;
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) offset += wave_count[w];
+      total += wave_count[w];
+    }
+    if (mine) list[(size_t)e * capacity + offset + before] = p;
+    base += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) counts[e] = base;
+}
+
+extern "C" int bh_experts_group(const int32_t* chosen, int n_pairs, int32_t* list, int capacity, int32_t* counts, int E, hipStream_t stream) {
+  BH_REQUIRE(n_pairs > 0 && E > 0 && capacity > 0, "experts_group: sizes must be positive");
+  experts_group_kernel<<<E, 256, 0, stream>>>(chosen, n_pairs, list, capacity, counts);
+  return bh_check_launch("experts_group");
+}
+
+template <typename T>
+__device__ inline void load8(const T* __restrict__ p, float (&v)[8]);
+template <>
+__device__ inline void load8<float>(const float* __restrict__ p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+template <>
+__device__ inline void load8<bf16_t>(const bf16_t* __restrict__ p, float (&v)[8]) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = bf16_bits_to_f32((uint16_t)(w[i] & 0xffffu));
+    v[2 * i + 1] = bf16_bits_to_f32((uint16_t)(w[i] >> 16));
+  }
+}
+
+#define ER_PAIRS 8      // pairs whose sums a wave keeps at a time
+#define ER_OUTS 16      // outputs a workgroup computes
+
+// grid (E, ceil(N / ER_OUTS)).  in [*][K]: the input of pair p is row p / in_div.  w [E][GATED ? 2 N : N][K].
+// GATED: out (T) [pairs][N] = act(gate row . x, up row . x);  otherwise out (float) [pairs][N] = row . x.
+// A wave takes U outputs at a time, so that the loads of U (gated: 2 U) weight rows are in flight together.
+// K must be a multiple of 8 (16-byte loads).
+template <typename T, bool GATED, int U>
+__global__ __launch_bounds__(256) void experts_rows_kernel(const T* __restrict__ in, int in_div, const int32_t* __restrict__ list, int capacity,
+                                                           const int32_t* __restrict__ counts, const T* __restrict__ w, void* __restrict__ out_raw,
+                                                           int K, int N, float limit, float alpha) {
+  const int e = blockIdx.x, count = counts[e];
+  if (count == 0) return;
+  const int lane = threadIdx.x & (BH_WAVE - 1), wave = threadIdx.x / BH_WAVE;
+  const int32_t* mine = list + (size_t)e * capacity;
+  const T* base = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+  for (int i = wave * U; i < ER_OUTS; i += 4 * U) {
+    const int o0 = blockIdx.y * ER_OUTS + i;
+    if (o0 >= N) break;
+    const T* row_a[U];
+    const T* row_b[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int o = o0 + u < N ? o0 + u : N - 1;      // a row beyond the last is computed again and not stored
+      row_a[u] = base + (size_t)o * K;
+      row_b[u] = base + (size_t)(N + o) * K;
+    }
+    for (int p0 = 0; p0 < count; p0 += ER_PAIRS) {
+      const int n_pairs = count - p0 < ER_PAIRS ? count - p0 : ER_PAIRS;
+      const T* x[ER_PAIRS];
+#pragma unroll
+      for (int j = 0; j < ER_PAIRS; ++j) x[j] = in + (size_t)(mine[p0 + (j < n_pairs ? j : 0)] / in_div) * K;
+      float acc_a[U][ER_PAIRS] = {}, acc_b[U][ER_PAIRS] = {};
+      for (int k = lane * 8; k < K; k += BH_WAVE * 8) {
+        float wa[U][8], wb[U][8], xv[8];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          load8<T>(row_a[u] + k, wa[u]);
+          if (GATED) load8<T>(row_b[u] + k, wb[u]);
+        }
+#pragma unroll
+        for (int j = 0; j < ER_PAIRS; ++j) {
+          if (j < n_pairs) {
+            load8<T>(x[j] + k, xv);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+              for (int t = 0; t < 8; ++t) {
+                acc_a[u][j] = fmaf(wa[u][t], xv[t], acc_a[u][j]);
+                if (GATED) acc_b[u][j] = fmaf(wb[u][t], xv[t], acc_b[u][j]);
+              }
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < ER_PAIRS; ++j) {
+        if (j >= n_pairs) break;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const float a = wave_sum(acc_a[u][j]);
+          const float b = GATED ? wave_sum(acc_b[u][j]) : 0.f;
+          if (lane == 0 && o0 + u < N) {
+            const size_t at = (size_t)mine[p0 + j] * N + o0 + u;
+            if (GATED) reinterpret_cast<T*>(out_raw)[at] = from_f32<T>(clamped_glu(a, b, limit, alpha));
+            else reinterpret_cast<float*>(out_raw)[at] = a;
+          }
+        }
+      }
+    }
+  }
+}
+
+extern "C" int bh_experts_rows(const void* in, int dtype, int in_div, const int32_t* list, int capacity, const int32_t* counts, const void* w,
+                               void* out, int E, int K, int N, int gated, float limit, float alpha, hipStream_t stream) {
+  BH_REQUIRE(E > 0 && K > 0 && N > 0 && in_div > 0 && capacity > 0, "experts_rows: sizes must be positive");
+  BH_REQUIRE(K % 8 == 0, "experts_rows: rows of a multiple of 8 inputs, got %d", K);
+  dim3 grid(E, (N + ER_OUTS - 1) / ER_OUTS);
+#define BH_ER(T, G, U) experts_rows_kernel<T, G, U><<<grid, 256, 0, stream>>>((const T*)in, in_div, list, capacity, counts, (const T*)w, out, K, N, limit, alpha)
+  if (dtype == BH_F32) {
+    if (gated) BH_ER(float, true, 2);
+    else BH_ER(float, false, 4);
+  } else if (dtype == BH_BF16) {
+    if (gated) BH_ER(bf16_t, true, 2);
+    else BH_ER(bf16_t, false, 4);
+  } else {
+    return bh_fail("experts_rows: unknown dtype %d", dtype);
+  }
+#undef BH_ER
+  return bh_check_launch("experts_rows");
+}
+
+// grid (E, rows of the grid's second axis walk an expert's pairs).  offsets [E]: where an expert's rows start in `sorted`.
+template <typename T>
+__global__ __launch_bounds__(256) void experts_gather_kernel(const T* __restrict__ x, int top, const int32_t* __restrict__ list, int capacity,
+                                                             const int32_t* __restrict__ counts, const int32_t* __restrict__ offsets,
+                                                             T* __restrict__ sorted, int32_t* __restrict__ place, int K) {
+  const int e = blockIdx.x, count = counts[e], first = offsets[e];
+  for (int i = blockIdx.y; i < count; i += gridDim.y) {
+    const int pair = list[(size_t)e * capacity + i];
+    const T* from = x + (size_t)(pair / top) * K;
+    T* to = sorted + (size_t)(first + i) * K;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) to[k] = from[k];
+    if (threadIdx.x == 0) place[pair] = first + i;
+  }
+}
+
+extern "C" int bh_experts_gather(const void* x, int dtype, int top, const int32_t* list, int capacity, const int32_t* counts,
+                                 const int32_t* offsets, void* sorted, int32_t* place, int E, int K, int n_rows, hipStream_t stream) {
+  BH_REQUIRE(E > 0 && K > 0 && top > 0 && n_rows > 0, "experts_gather: sizes must be positive");
+  dim3 grid(E, n_rows < 256 ? n_rows : 256);
+  if (dtype == BH_F32)
+    experts_gather_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, top, list, capacity, counts, offsets, (float*)sorted, place, K);
+  else if (dtype == BH_BF16)
+    experts_gather_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, top, list, capacity, counts, offsets, (bf16_t*)sorted, place, K);
+  else
+    return bh_fail("experts_gather: unknown dtype %d", dtype);
+  return bh_check_launch("experts_gather");
+}
+
+// y [*][D] float32: the result of pair p lies at row place[p] (or p where no places are given).
+__global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ place,
+                                                              const float* __restrict__ weights, float* __restrict__ hidden, int top, int D) {
+  const int row = blockIdx.x;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float total = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const int pair = row * top + j;
+      total = fmaf(weights[pair], y[(size_t)(place ? place[pair] : pair) * D + d], total);
+    }
+    hidden[(size_t)row * D + d] += total;
+  }
+}
+
+extern "C" int bh_experts_combine(const float* y, const int32_t* place, const float* weights, float* hidden, int n_rows, int top, int D,
+                                  hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && top > 0 && D > 0, "experts_combine: sizes must be positive");
+  experts_combine_kernel<<<n_rows, 256, 0, stream>>>(y, place, weights, hidden, top, D);
+  return bh_check_launch("experts_combine");
 }

@@ -98,6 +98,218 @@ extern "C" int bh_ssm_scan(const float* xbc, int xbc_stride, const void* proj, i
   return bh_check_launch("ssm_scan");
 }
 
+// ---- the same recurrence with the state in registers ------------------------------------------------------------
+// Thread (p, s) keeps its NPT state rows of column p in registers; SS_STAGE rows of B, C, x and the step sizes go through
+// LDS at a time, and the slices' shares of those rows' outputs are added in slice order.  A long sequence is cut into
+// chunks of rows that run side by side:
+//   MODE 1  every chunk walks its rows from a zero state, leaves its rows' outputs, its final state and, for every row,
+//           the logarithm of the decay from the chunk's start up to and including that row
+//   ssm_combine  goes through a sequence's chunks in order: the state a chunk truly starts from replaces the chunk's own
+//           in the scratch memory, and the state after the last chunk goes to the sequence's region
+//   MODE 2  every chunk adds to its rows what its true starting state owes them: y_t += exp(cum_t) S_in^T C_t
+// MODE 0 is a sequence in one piece, from and to its region (decode steps, short prompts).
+#define SS_STAGE 16
+
+template <typename T, int NPT, int MODE>
+__global__ __launch_bounds__(256) void ssm_chunk_kernel(const float* __restrict__ xbc, int xbc_stride, const T* __restrict__ proj,
+                                                        int proj_stride, int dt_first, const float* __restrict__ dt_bias,
+                                                        const float* __restrict__ a_log, const float* __restrict__ d_skip,
+                                                        float* __restrict__ state, long slot_stride, float* __restrict__ chunk_states,
+                                                        float* __restrict__ chunk_decay, float* __restrict__ cum,
+                                                        const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
+                                                        float* __restrict__ y, int H, int vdim, int N, int G, int slices, int chunk_rows,
+                                                        int chunks_per_seq) {
+  extern __shared__ float lds[];
+  float* bc = lds;                                 // [SS_STAGE][2 N]: B, C of a row
+  float* xs = bc + SS_STAGE * 2 * N;               // [SS_STAGE][vdim]
+  float* part = xs + SS_STAGE * vdim;              // [SS_STAGE][slices][vdim]
+  float* fac = part + SS_STAGE * slices * vdim;    // [SS_STAGE][2]: log decay (MODE 2: the decay since the chunk's start), dt
+  const int seq = blockIdx.x / chunks_per_seq, chunk = blockIdx.x % chunks_per_seq, head = blockIdx.y;
+  const int seq_stop = seq_start[seq + 1];
+  const int start = seq_start[seq] + chunk * chunk_rows;
+  if (start >= seq_stop) return;
+  const int stop = start + chunk_rows < seq_stop ? start + chunk_rows : seq_stop;
+  const int group = head / (H / G), inner = H * vdim;
+  const int p = threadIdx.x % vdim, s = threadIdx.x / vdim;
+  const bool works = s < slices;
+  const int per = (N + slices - 1) / slices;
+  const int n0 = s * per, n1 = n0 + per < N ? n0 + per : N;
+  float* home = MODE == 0 ? state + (size_t)seq_slot[seq] * slot_stride + (size_t)head * N * vdim
+                          : chunk_states + ((size_t)blockIdx.x * H + head) * N * vdim;
+  float S[NPT];
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) S[i] = (MODE != 1 && works && n0 + i < n1) ? home[(size_t)(n0 + i) * vdim + p] : 0.f;
+  const float rate = expf(a_log[head]), skip = d_skip[head], bias = dt_bias[head];
+  float run = 0.f;
+  for (int r0 = start; r0 < stop; r0 += SS_STAGE) {
+    const int rows = stop - r0 < SS_STAGE ? stop - r0 : SS_STAGE;
+    for (int e = threadIdx.x; e < rows * 2 * N; e += blockDim.x) {
+      const int r = e / (2 * N), j = e % (2 * N);
+      bc[r * 2 * N + j] = xbc[(size_t)(r0 + r) * xbc_stride + inner + (j < N ? group * N + j : (G + group) * N + j - N)];
+    }
+    for (int e = threadIdx.x; e < rows * vdim; e += blockDim.x)
+      xs[e] = xbc[(size_t)(r0 + e / vdim) * xbc_stride + head * vdim + e % vdim];
+    if (threadIdx.x < rows) {
+      if (MODE == 2) {
+        fac[2 * threadIdx.x] = expf(cum[(size_t)(r0 + threadIdx.x) * H + head]);
+      } else {
+        const float dt = softplus_f32(to_f32(proj[(size_t)(r0 + threadIdx.x) * proj_stride + dt_first + head]) + bias);
+        fac[2 * threadIdx.x] = -rate * dt;
+        fac[2 * threadIdx.x + 1] = dt;
+      }
+    }
+    __syncthreads();
+    if (MODE == 1 && threadIdx.x == 0) {
+      for (int r = 0; r < rows; ++r) {
+        run += fac[2 * r];
+        cum[(size_t)(r0 + r) * H + head] = run;
+      }
+    }
+    if (works) {
+      for (int r = 0; r < rows; ++r) {
+        const float* b = bc + r * 2 * N;
+        const float* c = b + N;
+        float acc = 0.f;
+        if (MODE == 2) {
+#pragma unroll
+          for (int i = 0; i < NPT; ++i)
+            if (n0 + i < n1) acc = fmaf(S[i], c[n0 + i], acc);
+        } else {
+          const float decay = expf(fac[2 * r]), dtx = fac[2 * r + 1] * xs[r * vdim + p];
+#pragma unroll
+          for (int i = 0; i < NPT; ++i) {
+            if (n0 + i < n1) {
+              S[i] = fmaf(decay, S[i], b[n0 + i] * dtx);
+              acc = fmaf(S[i], c[n0 + i], acc);
+            }
+          }
+        }
+        part[(r * slices + s) * vdim + p] = acc;
+      }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < rows * vdim; e += blockDim.x) {
+      const int r = e / vdim, i = e % vdim;
+      float total = 0.f;
+      for (int k = 0; k < slices; ++k) total += part[(r * slices + k) * vdim + i];
+      float* out = y + (size_t)(r0 + r) * inner + head * vdim + i;
+      if (MODE == 2) *out += fac[2 * r] * total;
+      else *out = total + skip * xs[e];
+    }
+    __syncthreads();
+  }
+  if (MODE != 2 && works) {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      if (n0 + i < n1) home[(size_t)(n0 + i) * vdim + p] = S[i];
+  }
+  if (MODE == 1 && threadIdx.x == 0) chunk_decay[(size_t)blockIdx.x * H + head] = run;
+}
+
+// grid (sequences, heads): a thread per state element walks the sequence's chunks in order.
+__global__ __launch_bounds__(256) void ssm_combine_kernel(float* __restrict__ state, long slot_stride, float* __restrict__ chunk_states,
+                                                          const float* __restrict__ chunk_decay, const int32_t* __restrict__ seq_start,
+                                                          const int32_t* __restrict__ seq_slot, int H, int elements, int chunk_rows,
+                                                          int chunks_per_seq) {
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int n_rows = seq_start[seq + 1] - seq_start[seq];
+  const int chunks = (n_rows + chunk_rows - 1) / chunk_rows;
+  float* home = state + (size_t)seq_slot[seq] * slot_stride + (size_t)head * elements;
+  for (int e = threadIdx.x; e < elements; e += blockDim.x) {
+    float S = home[e];
+    for (int c = 0; c < chunks; ++c) {
+      const size_t at = (size_t)seq * chunks_per_seq + c;
+      float* slot = chunk_states + (at * H + head) * elements + e;
+      const float local = *slot;
+      *slot = S;
+      S = fmaf(expf(chunk_decay[at * H + head]), S, local);
+    }
+    home[e] = S;
+  }
+}
+
+// How a step's sequences are cut: rows a chunk (a multiple of SS_STAGE) for sequences of up to max_rows rows, so that the
+// chip has about two workgroups a compute unit where the rows allow it, and no chunk is shorter than 64 rows.
+extern "C" int bh_ssm_chunk_rows(int n_seqs, int max_rows, int H) {
+  if (max_rows <= 128) return max_rows < 1 ? 1 : max_rows;
+  long wanted = (2L * bh_compute_units() + (long)n_seqs * H - 1) / ((long)n_seqs * H);
+  const int most = max_rows / 64;
+  if (wanted > most) wanted = most;
+  if (wanted < 1) wanted = 1;
+  const int rows = (int)((max_rows + wanted - 1) / wanted);
+  return (rows + SS_STAGE - 1) / SS_STAGE * SS_STAGE;
+}
+
+// Whether the recurrence with the state in registers takes these sizes (otherwise bh_ssm_scan walks with the state in LDS).
+extern "C" int bh_ssm_fast_takes(int vdim, int N) {
+  if (vdim > 256 || vdim < 1 || N < 1) return 0;
+  int slices = 256 / vdim;
+  if (slices > N) slices = N;
+  const int per = (N + slices - 1) / slices;
+  const size_t lds = ((size_t)SS_STAGE * (2 * N + vdim + slices * vdim + 2)) * sizeof(float);
+  return per <= 128 && lds <= 150 * 1024;
+}
+
+template <typename T, int NPT>
+static int ssm_fast_launch(const float* xbc, int xbc_stride, const T* proj, int proj_stride, int dt_first, const float* dt_bias,
+                           const float* a_log, const float* d_skip, float* state, long slot_stride, float* chunk_states,
+                           float* chunk_decay, float* cum, const int32_t* seq_start, const int32_t* seq_slot, float* y, int n_seqs, int H,
+                           int vdim, int N, int G, int slices, int chunk_rows, int chunks_per_seq, size_t lds, hipStream_t stream) {
+  dim3 grid(n_seqs * chunks_per_seq, H);
+#define BH_SS(MODE)                                                                                                                 \
+  do {                                                                                                                              \
+    if (lds > 48 * 1024)                                                                                                            \
+      (void)hipFuncSetAttribute((const void*)ssm_chunk_kernel<T, NPT, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+    ssm_chunk_kernel<T, NPT, MODE><<<grid, 256, lds, stream>>>(xbc, xbc_stride, proj, proj_stride, dt_first, dt_bias, a_log, d_skip,   \
+                                                               state, slot_stride, chunk_states, chunk_decay, cum, seq_start, seq_slot, \
+                                                               y, H, vdim, N, G, slices, chunk_rows, chunks_per_seq);                \
+  } while (0)
+  if (chunks_per_seq == 1) {
+    BH_SS(0);
+    return bh_check_launch("ssm_scan");
+  }
+  BH_SS(1);
+  ssm_combine_kernel<<<dim3(n_seqs, H), 256, 0, stream>>>(state, slot_stride, chunk_states, chunk_decay, seq_start, seq_slot, H, N * vdim,
+                                                         chunk_rows, chunks_per_seq);
+  BH_SS(2);
+#undef BH_SS
+  return bh_check_launch("ssm_scan in chunks");
+}
+
+// chunk_states [n_seqs * chunks_per_seq][H][N][vdim], chunk_decay [n_seqs * chunks_per_seq][H] and cum [rows][H] are scratch
+// memory of the call (unused, and may be null, with one chunk a sequence).
+extern "C" int bh_ssm_scan_fast(const float* xbc, int xbc_stride, const void* proj, int dtype, int proj_stride, int dt_first,
+                                const float* dt_bias, const float* a_log, const float* d_skip, float* state, long slot_stride,
+                                float* chunk_states, float* chunk_decay, float* cum, const int32_t* seq_start, const int32_t* seq_slot,
+                                float* y, int n_seqs, int H, int vdim, int N, int G, int chunk_rows, int chunks_per_seq,
+                                hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && H > 0 && G > 0 && H % G == 0, "ssm_scan: %d heads in %d groups", H, G);
+  BH_REQUIRE(bh_ssm_fast_takes(vdim, N), "ssm_scan: the form with the state in registers does not take heads of %d with %d rows", vdim, N);
+  BH_REQUIRE(xbc_stride >= H * vdim + 2 * G * N, "ssm_scan: a row of %d does not hold x, B and C", xbc_stride);
+  BH_REQUIRE(dt_first >= 0 && dt_first + H <= proj_stride, "ssm_scan: the step sizes lie outside their row");
+  BH_REQUIRE(chunk_rows > 0 && chunks_per_seq > 0 && (chunks_per_seq == 1 || (chunk_rows % SS_STAGE == 0 && chunk_states && chunk_decay && cum)),
+             "ssm_scan: chunks of a multiple of %d rows with their scratch memory", SS_STAGE);
+  int slices = 256 / vdim;
+  if (slices > N) slices = N;
+  const int per = (N + slices - 1) / slices;
+  const size_t lds = ((size_t)SS_STAGE * (2 * N + vdim + slices * vdim + 2)) * sizeof(float);
+#define BH_SF(T, NPT)                                                                                                              \
+  return ssm_fast_launch<T, NPT>(xbc, xbc_stride, (const T*)proj, proj_stride, dt_first, dt_bias, a_log, d_skip, state, slot_stride, \
+                                 chunk_states, chunk_decay, cum, seq_start, seq_slot, y, n_seqs, H, vdim, N, G, slices, chunk_rows,   \
+                                 chunks_per_seq, lds, stream)
+  if (dtype == BH_F32) {
+    if (per <= 8) BH_SF(float, 8);
+    if (per <= 32) BH_SF(float, 32);
+    BH_SF(float, 128);
+  } else if (dtype == BH_BF16) {
+    if (per <= 8) BH_SF(bf16_t, 8);
+    if (per <= 32) BH_SF(bf16_t, 32);
+    BH_SF(bf16_t, 128);
+  }
+#undef BH_SF
+  return bh_fail("ssm_scan: unknown dtype %d", dtype);
+}
+
 // One workgroup a (row, group).
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_stride,

@@ -6,6 +6,7 @@
 //                           position * freq[i]; q into a matrix of heads of `pad` dimensions, k and v into the cache
 //                           pages of (sequence, position) as heads of `pad` (zeros beyond dim and vdim), so that keys of
 //                           one size and values of another go through kernels that know one head size
+//   conv_norm_rope_write    the same from the projected rows, the short convolution made on the way
 //   gate_heads              out[row][h][i] = attended[row][h][i] * sigmoid(gate[row][h][i]) for i < vdim
 // Statistics, angles, cosines and sines are float32; the angle is the float32 product position * freq[i].
 #include "common.h"
@@ -90,6 +91,119 @@ extern "C" int bh_whole_norm_rope_write(const float* qkv, const float* wq, const
   else
     return bh_fail("whole_norm_rope_write: unknown dtype %d", dtype);
   return bh_check_launch("whole_norm_rope_write");
+}
+
+// The same from the projected rows themselves: the short convolution over time (csrc/short_conv.hip has its definition and
+// its state) is made on the way, a row's convolved channels stand in LDS as float32 and are never written to memory.
+// proj [n_rows][row_stride]: a row holds, from `first`, q, k and v; w_conv [q + k + v channels][taps] (taps 0: no convolution).
+template <typename T>
+__global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
+    const T* __restrict__ proj, int row_stride, int first, const float* __restrict__ w_conv, int taps, const float* __restrict__ state,
+    long slot_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ row_seq, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    const int32_t* __restrict__ page_table, int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write) {
+  extern __shared__ float conv[];      // [q | k | v] of this row
+  __shared__ float scratch[8];
+  const int row = blockIdx.x;
+  const int q_width = H * dim, k_width = G * dim, v_width = G * vdim, channels = q_width + k_width + v_width;
+  const int seq = row_seq[row], pos = positions[row];
+  const int t = row - seq_start[seq];
+  const float* old = state ? state + (size_t)seq_slot[seq] * slot_stride : nullptr;
+  float ss_q = 0.f, ss_k = 0.f;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float acc;
+    if (taps <= 1) {
+      acc = to_f32(proj[(size_t)row * row_stride + first + c]) * (taps ? w_conv[c] : 1.f);
+    } else {
+      acc = 0.f;
+      for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;
+        const float u = back <= t ? to_f32(proj[(size_t)(row - back) * row_stride + first + c])
+                                  : old[(size_t)(taps - 1 + t - back) * channels + c];
+        acc = fmaf(w_conv[(size_t)c * taps + j], u, acc);
+      }
+    }
+    conv[c] = acc;
+    if (c < q_width) ss_q += acc * acc;
+    else if (c < q_width + k_width) ss_k += acc * acc;
+  }
+  const float inv_q = 1.0f / sqrtf(block_sum(ss_q, scratch) / (float)q_width + eps);
+  const float inv_k = 1.0f / sqrtf(block_sum(ss_k, scratch) / (float)k_width + eps);
+  const float* q = conv;
+  const float* k = conv + q_width;
+  const float* v = k + k_width;
+  for (int e = threadIdx.x; e < H * pad; e += blockDim.x) {
+    const int head = e / pad, i = e % pad;
+    float y = 0.f;
+    if (i < dim) {
+      const int at = head * dim + i;
+      y = q[at] * inv_q * wq[at];
+      if (i < turned) {
+        const int mate = at ^ 1;
+        const float other = q[mate] * inv_q * wq[mate];
+        const float angle = (float)pos * freq[i >> 1];
+        const float c = cosf(angle), s = sinf(angle);
+        y = (i & 1) ? y * c + other * s : y * c - other * s;
+      }
+    }
+    q_out[(size_t)row * H * pad + e] = from_f32<T>(y);
+  }
+  if (!write) return;
+  const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE], token = pos % BH_PAGE;
+  for (int e = threadIdx.x; e < G * pad; e += blockDim.x) {
+    const int head = e / pad, i = e % pad;
+    float y = 0.f;
+    if (i < dim) {
+      const int at = head * dim + i;
+      y = k[at] * inv_k * wk[at];
+      if (i < turned) {
+        const int mate = at ^ 1;
+        const float other = k[mate] * inv_k * wk[mate];
+        const float angle = (float)pos * freq[i >> 1];
+        const float c = cosf(angle), s = sinf(angle);
+        y = (i & 1) ? y * c + other * s : y * c - other * s;
+      }
+    }
+    T* keys = k_pages + ((size_t)page * G + head) * BH_PAGE * pad;
+    T* values = v_pages + ((size_t)page * G + head) * BH_PAGE * pad;
+    keys[bh_key_index(kv_order, token, i, pad)] = from_f32<T>(y);
+    values[bh_value_index(kv_order, token, i, pad)] = from_f32<T>(i < vdim ? v[head * vdim + i] : 0.f);
+  }
+}
+
+extern "C" int bh_conv_norm_rope_write(const void* proj, int dtype, int row_stride, int first, const float* w_conv, int taps,
+                                       const float* state, long slot_stride, const int32_t* seq_start, const int32_t* seq_slot,
+                                       const float* wq, const float* wk, float eps, const float* freq, int turned,
+                                       const int32_t* positions, const int32_t* row_seq, void* q_out, void* k_pages, void* v_pages,
+                                       const int32_t* page_table, int table_stride, int n_rows, int H, int G, int dim, int vdim, int pad,
+                                       int kv_order, int write, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && G > 0 && dim > 0 && vdim > 0, "conv_norm_rope_write: sizes must be positive");
+  BH_REQUIRE(pad >= dim && pad >= vdim, "conv_norm_rope_write: heads of %d do not hold keys of %d and values of %d", pad, dim, vdim);
+  BH_REQUIRE(turned == 0 || (turned % 2 == 0 && turned <= dim && dim % 2 == 0 && freq != nullptr),
+             "conv_norm_rope_write: %d turned dimensions of %d", turned, dim);
+  BH_REQUIRE(taps >= 0 && taps <= 16 && (taps <= 1 || state != nullptr) && (taps == 0 || w_conv != nullptr),
+             "conv_norm_rope_write: %d taps need their weights and, beyond one, a state", taps);
+  const int channels = (H + G) * dim + G * vdim;
+  BH_REQUIRE(first >= 0 && first + channels <= row_stride, "conv_norm_rope_write: q, k and v lie outside a row of %d", row_stride);
+  BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && pad % 32 == 0),
+             "conv_norm_rope_write: cache order %d does not exist for head size %d", kv_order, pad);
+  const size_t lds = (size_t)channels * sizeof(float);
+  BH_REQUIRE(lds <= 128 * 1024, "conv_norm_rope_write: %d channels do not fit the local memory", channels);
+#define BH_CW(T)                                                                                                                   \
+  do {                                                                                                                             \
+    if (lds > 48 * 1024)                                                                                                           \
+      (void)hipFuncSetAttribute((const void*)conv_norm_rope_write_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    conv_norm_rope_write_kernel<T><<<n_rows, 256, lds, stream>>>((const T*)proj, row_stride, first, w_conv, taps, state, slot_stride,  \
+                                                                 seq_start, seq_slot, wq, wk, eps, freq, turned, positions, row_seq, \
+                                                                 (T*)q_out, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, G, \
+                                                                 dim, vdim, pad, kv_order, write);                                  \
+  } while (0)
+  if (dtype == BH_F32) BH_CW(float);
+  else if (dtype == BH_BF16) BH_CW(bf16_t);
+  else return bh_fail("conv_norm_rope_write: unknown dtype %d", dtype);
+#undef BH_CW
+  return bh_check_launch("conv_norm_rope_write");
 }
 
 template <typename T>

@@ -188,6 +188,14 @@ class KernelSizes:
             "bh_experts_gate_up": [p, i, p, p, p, i, i, i, i, f, f, p],
             "bh_experts_down": [p, i, p, p, p, p, i, i, i, i, p],
             "bh_clamped_glu": [p, i, p, i, i, f, f, i, p],
+            "bh_conv_norm_rope_write": [p, i, i, i, p, i, p, ctypes.c_long, p, p, p, p, f, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
+            "bh_ssm_scan_fast": [p, i, p, i, i, i, p, p, p, p, ctypes.c_long, p, p, p, p, p, p, i, i, i, i, i, i, i, p],
+            "bh_ssm_chunk_rows": [i, i, i],
+            "bh_ssm_fast_takes": [i, i],
+            "bh_experts_group": [p, i, p, i, p, i, p],
+            "bh_experts_rows": [p, i, i, p, i, p, p, p, i, i, i, i, f, f, p],
+            "bh_experts_gather": [p, i, i, p, i, p, p, p, p, i, i, i, p],
+            "bh_experts_combine": [p, p, p, p, i, i, i, p],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
@@ -1046,6 +1054,36 @@ class HipKernels(KernelSizes):
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
             self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
 
+    def conv_norm_rope_write(self, proj, first, conv_weight, state, state_offset, seq_start, seq_slot, q_weight, k_weight, eps, freq,
+                             turned, positions, row_seq, q_out, k_pages, v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+        """`short_conv` of the q, k, v channels of `proj` (from column `first`; conv_weight f32 [channels, taps], or None for no
+        convolution) and `whole_norm_rope_write` of the result in one launch: the convolved row is never written to memory.  The
+        state is read, not updated (`short_conv_state` afterwards)."""
+        n_rows = proj.shape[0]
+        channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
+        taps = conv_weight.shape[1] if conv_weight is not None else 0
+        if tuple(q_out.shape) != (n_rows, n_heads * pad) or q_out.dtype != proj.dtype or (conv_weight is not None and conv_weight.shape[0] != channels):
+            raise KernelError(f"conv_norm_rope_write: shapes proj {tuple(proj.shape)}, q_out {tuple(q_out.shape)} do not fit")
+        if q_weight.shape != (n_heads * dim,) or k_weight.shape != (n_kv_heads * dim,):
+            raise KernelError("conv_norm_rope_write: one norm weight per query channel and per key channel")
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,) or seq_start.shape != (seq_slot.shape[0] + 1,):
+            raise KernelError("conv_norm_rope_write: positions and row_seq have one entry per row, seq_start one per sequence and one more")
+        if turned and (freq is None or freq.shape != (turned // 2,)):
+            raise KernelError("conv_norm_rope_write: one frequency per turned pair")
+        where, stride = None, 0
+        if taps > 1:
+            where, stride = self._state_view(state, state_offset, (taps - 1) * channels, "conv_norm_rope_write")
+            self._ptr(state, "conv state", (torch.float32,))
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, pad, q_out.dtype, "conv_norm_rope_write")
+        self._check(self.lib.bh_conv_norm_rope_write(
+            self._ptr(proj, "proj"), _code(proj, "proj"), proj.shape[1], int(first), self._ptr(conv_weight, "conv weight", (torch.float32,), True),
+            taps, where, stride, self._ptr(seq_start, "seq_start", (torch.int32,)), self._ptr(seq_slot, "seq_slot", (torch.int32,)),
+            self._ptr(q_weight, "q norm", (torch.float32,)), self._ptr(k_weight, "k norm", (torch.float32,)), float(eps),
+            self._ptr(freq, "frequencies", (torch.float32,), True), int(turned), self._ptr(positions, "positions", (torch.int32,)),
+            self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(q_out, "q_out"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
+            self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
+
     def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim):
         """out[r, h, i] = attended[r, h, i] * sigmoid(gate[r, gate_first + h vdim + i]), i < vdim; attended [n, H pad]."""
         n_rows = attended.shape[0]
@@ -1057,11 +1095,23 @@ class HipKernels(KernelSizes):
             gate.shape[1], int(gate_first), self._ptr(out, "gate_heads out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
 
     # ---- a state-space recurrence with a scalar decay per head ----
+    def ssm_chunk_bytes(self, n_seqs, n_rows, max_rows, n_heads, vdim, n_state) -> int:
+        """Bytes of scratch memory that `ssm_scan` allocates for a step of these sizes (sequences cut into chunks)."""
+        if not self.lib.bh_ssm_fast_takes(int(vdim), int(n_state)):
+            return 0
+        chunk_rows = int(self.lib.bh_ssm_chunk_rows(int(n_seqs), int(max_rows), int(n_heads)))
+        chunks = -(-int(max_rows) // chunk_rows)
+        if chunks <= 1:
+            return 0
+        return (_rounded(n_seqs * chunks * n_heads * n_state * vdim * 4) + _rounded(n_seqs * chunks * n_heads * 4)
+                + _rounded(n_rows * n_heads * 4))
+
     def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
-                 n_state, n_groups):
+                 n_state, n_groups, max_rows_per_seq=None):
         """Per (sequence, head): S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x with dt = softplus(proj[:, dt_first
         + head] + dt_bias); xbc f32 [n, H vdim + 2 G N] = [x | B | C], S [H, N, vdim] f32 at `state_offset` floats into
-        state[slot], out f32 [n, H vdim]."""
+        state[slot], out f32 [n, H vdim].  `max_rows_per_seq` (the most rows any sequence brings; the step's rows if not
+        given) decides whether long sequences are cut into chunks that run side by side."""
         n_rows, n_seqs = xbc.shape[0], seq_slot.shape[0]
         inner = n_heads * vdim
         if xbc.shape != (n_rows, inner + 2 * n_groups * n_state) or tuple(out.shape) != (n_rows, inner) or proj.shape[0] != n_rows:
@@ -1070,12 +1120,25 @@ class HipKernels(KernelSizes):
             raise KernelError("ssm_scan: one dt_bias, A_log and D per head, and seq_start with one entry per sequence and one more")
         where, stride = self._state_view(state, state_offset, n_heads * n_state * vdim, "ssm_scan")
         self._ptr(state, "ssm_scan state", (torch.float32,))
-        self._check(self.lib.bh_ssm_scan(
-            self._ptr(xbc, "ssm_scan xbc", (torch.float32,)), xbc.shape[1], self._ptr(proj, "ssm_scan proj"), _code(proj, "ssm_scan proj"),
-            proj.shape[1], int(dt_first), self._ptr(dt_bias, "dt_bias", (torch.float32,)), self._ptr(a_log, "A_log", (torch.float32,)),
-            self._ptr(d_skip, "D", (torch.float32,)), where, stride, self._ptr(seq_start, "seq_start", (torch.int32,)),
-            self._ptr(seq_slot, "seq_slot", (torch.int32,)), self._ptr(out, "ssm_scan out", (torch.float32,)), n_seqs, n_heads, vdim,
-            n_state, n_groups, self._stream()))
+        common = (self._ptr(xbc, "ssm_scan xbc", (torch.float32,)), xbc.shape[1], self._ptr(proj, "ssm_scan proj"), _code(proj, "ssm_scan proj"),
+                  proj.shape[1], int(dt_first), self._ptr(dt_bias, "dt_bias", (torch.float32,)), self._ptr(a_log, "A_log", (torch.float32,)),
+                  self._ptr(d_skip, "D", (torch.float32,)), where, stride)
+        rest = (self._ptr(seq_start, "seq_start", (torch.int32,)), self._ptr(seq_slot, "seq_slot", (torch.int32,)),
+                self._ptr(out, "ssm_scan out", (torch.float32,)), n_seqs, n_heads, vdim, n_state, n_groups)
+        if not self.lib.bh_ssm_fast_takes(int(vdim), int(n_state)):
+            self._check(self.lib.bh_ssm_scan(*common, *rest, self._stream()))
+            return
+        most = int(max_rows_per_seq) if max_rows_per_seq else n_rows
+        chunk_rows = int(self.lib.bh_ssm_chunk_rows(n_seqs, most, n_heads))
+        chunks = -(-most // chunk_rows)
+        states = decays = cum = None
+        if chunks > 1:
+            states = torch.empty((n_seqs * chunks, n_heads, n_state, vdim), dtype=torch.float32, device=self.device)
+            decays = torch.empty((n_seqs * chunks, n_heads), dtype=torch.float32, device=self.device)
+            cum = torch.empty((n_rows, n_heads), dtype=torch.float32, device=self.device)
+        self._check(self.lib.bh_ssm_scan_fast(
+            *common, self._ptr(states, "chunk states", None, True), self._ptr(decays, "chunk decays", None, True),
+            self._ptr(cum, "row decays", None, True), *rest, chunk_rows, chunks, self._stream()))
 
     def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups):
         """out = rms_g(y * silu(z[:, z_first : z_first + W])) * weight, the root mean square over each of `groups` equal
@@ -1125,6 +1188,57 @@ class HipKernels(KernelSizes):
             self._ptr(inner, "experts inner"), _code(inner, "experts inner"), self._ptr(chosen, "chosen", (torch.int32,)),
             self._ptr(weights, "route weights", (torch.float32,)), self._ptr(w_down, "expert down"),
             self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top, ff, width, self._stream()))
+
+    def experts_group(self, chosen, lists, counts):
+        """lists[e, :counts[e]] = the pairs p = row * top + j with chosen[row, j] == e, in ascending order; chosen int32 [n, top],
+        lists int32 [E, n], counts int32 [E]."""
+        n_rows, top = chosen.shape
+        experts = counts.shape[0]
+        if lists.shape != (experts, n_rows):
+            raise KernelError(f"experts_group: lists {tuple(lists.shape)} for {experts} experts and {n_rows} rows")
+        self._check(self.lib.bh_experts_group(self._ptr(chosen, "chosen", (torch.int32,)), n_rows * top, self._ptr(lists, "lists", (torch.int32,)),
+                                              n_rows, self._ptr(counts, "counts", (torch.int32,)), experts, self._stream()))
+
+    def experts_rows_take(self, inputs: int) -> bool:
+        """Whether `experts_rows` takes rows of that many inputs (16-byte loads)."""
+        return inputs % 8 == 0
+
+    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0):
+        """For every expert e and each of its pairs p (lists, counts): a product of w[e] with rows[p // rows_per_pair_row], the
+        expert's matrix read once per workgroup.  gated: w [E, 2 N, K] (gate rows, then up rows), out [pairs, N] of the rows' type
+        = act(gate, up); otherwise w [E, N, K] and out float32 [pairs, N]."""
+        experts, w_rows, k = w.shape
+        n = w_rows // 2 if gated else w_rows
+        if rows.shape[1] != k or out.shape[1] != n or w.dtype != rows.dtype or counts.shape != (experts,) or lists.shape[0] != experts \
+                or out.dtype != (rows.dtype if gated else torch.float32):
+            raise KernelError(f"experts_rows: shapes rows {tuple(rows.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_experts_rows(
+            self._ptr(rows, "experts rows"), _code(rows, "experts rows"), int(rows_per_pair_row), self._ptr(lists, "lists", (torch.int32,)),
+            lists.shape[1], self._ptr(counts, "counts", (torch.int32,)), self._ptr(w, "expert weights"), self._ptr(out, "experts out"),
+            experts, k, n, int(bool(gated)), float(limit), float(alpha), self._stream()))
+
+    def experts_gather(self, x, top, lists, counts, offsets, gathered, place):
+        """gathered[offsets[e] + i] = x[lists[e, i] // top] and place[lists[e, i]] = offsets[e] + i for i < counts[e]: the pairs'
+        input rows side by side, expert after expert."""
+        n_rows, k = x.shape
+        experts = counts.shape[0]
+        if tuple(gathered.shape) != (n_rows * top, k) or place.shape != (n_rows * top,) or offsets.shape != (experts,) \
+                or gathered.dtype != x.dtype:
+            raise KernelError(f"experts_gather: shapes x {tuple(x.shape)}, gathered {tuple(gathered.shape)} do not fit")
+        self._check(self.lib.bh_experts_gather(
+            self._ptr(x, "experts x"), _code(x, "experts x"), int(top), self._ptr(lists, "lists", (torch.int32,)), lists.shape[1],
+            self._ptr(counts, "counts", (torch.int32,)), self._ptr(offsets, "offsets", (torch.int32,)), self._ptr(gathered, "gathered"),
+            self._ptr(place, "place", (torch.int32,)), experts, k, n_rows, self._stream()))
+
+    def experts_combine(self, y, place, weights, hidden):
+        """hidden[r] += sum_j weights[r, j] * y[place[r * top + j]] (place None: y[r * top + j]), j in order; y f32 [pairs, D]."""
+        n_rows, top = weights.shape
+        if tuple(y.shape) != (n_rows * top, hidden.shape[1]) or hidden.shape[0] != n_rows or (place is not None and place.shape != (n_rows * top,)):
+            raise KernelError(f"experts_combine: shapes y {tuple(y.shape)}, hidden {tuple(hidden.shape)} do not fit")
+        self._check(self.lib.bh_experts_combine(
+            self._ptr(y, "experts y", (torch.float32,)), self._ptr(place, "place", (torch.int32,), True),
+            self._ptr(weights, "route weights", (torch.float32,)), self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top,
+            hidden.shape[1], self._stream()))
 
     def clamped_glu(self, gate_up, out, limit, alpha):
         """out = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit); gate_up [n, 2 ff] = [g | u]."""

@@ -98,16 +98,22 @@ class ConvGatedAttention:
         k = ctx.kernels
         n = ctx.n_rows
         proj = self.proj.forward(ctx, x)
-        conv = ctx.new_f32(n, self.conv_width)
         state = cache.state if self.taps > 1 else None
-        k.short_conv(proj, 0, self.conv_weight, None, state, 0, ctx.row_seq, ctx.seq_start, ctx.seq_slot, conv)
-        if state is not None and cache.writes:
-            k.short_conv_state(proj, 0, self.conv_width, self.taps, state, 0, ctx.seq_start, ctx.seq_slot)
         q = ctx.new_activations(n, self.n_heads * self.pad)
         freq = self.rotation.frequencies(ctx.device) if self.rotation is not None else None
-        k.whole_norm_rope_write(conv, self.q_norm, self.k_norm, self.norm_eps, freq, self.turned, ctx.positions, ctx.row_seq, q,
-                                cache.k_pages, cache.v_pages, cache.page_table, self.n_heads, self.n_kv_heads, self.dim, self.vdim,
-                                self.pad, cache.writes)
+        in_one = getattr(k, "conv_norm_rope_write", None)      # convolution, norm, rotation and cache write in one launch
+        if in_one is not None:
+            in_one(proj, 0, self.conv_weight if self.taps else None, state, 0, ctx.seq_start, ctx.seq_slot, self.q_norm, self.k_norm,
+                   self.norm_eps, freq, self.turned, ctx.positions, ctx.row_seq, q, cache.k_pages, cache.v_pages, cache.page_table,
+                   self.n_heads, self.n_kv_heads, self.dim, self.vdim, self.pad, cache.writes)
+        else:
+            conv = ctx.new_f32(n, self.conv_width)
+            k.short_conv(proj, 0, self.conv_weight, None, state, 0, ctx.row_seq, ctx.seq_start, ctx.seq_slot, conv)
+            k.whole_norm_rope_write(conv, self.q_norm, self.k_norm, self.norm_eps, freq, self.turned, ctx.positions, ctx.row_seq, q,
+                                    cache.k_pages, cache.v_pages, cache.page_table, self.n_heads, self.n_kv_heads, self.dim, self.vdim,
+                                    self.pad, cache.writes)
+        if state is not None and cache.writes:      # after every reader of the old state
+            k.short_conv_state(proj, 0, self.conv_width, self.taps, state, 0, ctx.seq_start, ctx.seq_slot)
         attended = ctx.new_activations(n, self.n_heads * self.pad)
         k.attention(q, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions, self.n_heads,
                     self.n_kv_heads, self.pad, self.scale, 0, layout=ctx)

@@ -6,9 +6,13 @@
     out = sum over chosen of weight * expert(h)  +  shared(h)        (the shared expert has the same form and runs for all)
 
 The experts' matrices are kept stacked: gate and up rows of an expert in one [2 ff, width] block, [experts, ...] in
-all.  A step of few rows reads a chosen expert's rows once per (row, expert) pair (`experts_gate_up`, `experts_down`),
-with no step that depends on the routing on the host, so that decode steps can be captured.  A row's result never
-depends on its batch-mates: its experts' shares are added in the order of its own choice.  The routing is left in
+all.  The (row, choice) pairs are grouped by expert on the device (`experts_group`).  A step of few rows then runs a
+workgroup per expert and block of outputs that reads the expert's rows from memory once for all of its pairs
+(`experts_rows`), with nothing that depends on the routing on the host, so that decode steps can be captured.  A step
+of many rows (a prompt) reads the experts' counts on the host (the step waits for the device there), lays the pairs'
+inputs side by side, expert after expert, and runs the framework's matrix products on each expert's stretch.  Sizes
+that the grouped kernels do not take go pair by pair (`experts_gate_up`, `experts_down`).  In every form a row's
+experts' shares are added in the order of its own choice, so its result depends on its batch-mates by rounding at most.  The routing is left in
 `ctx.extras["routing"]` ((chosen, weights) of the last layer that ran).  Every size and constant is a constructor
 parameter.
 """
@@ -63,7 +67,9 @@ class ClampedGLU:
 
 class RoutedExperts:
     graph_safe = True
-    graph_safe_rows = None
+    graph_safe_rows = 1       # steps of several rows a sequence may read the experts' counts on the host
+    PRODUCT_PAIRS = 16        # from that many pairs an expert on average, a step of many rows runs matrix products
+    PACK_FOR_PROMPTS = True   # keep a second copy of every expert's matrices in the form the products of many rows read fastest
 
     def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared: ClampedGLU | None = None,
                  alpha: float = GATE_SLOPE):
@@ -73,6 +79,7 @@ class RoutedExperts:
         self.limit, self.alpha, self.prefix, self.shared = float(limit), float(alpha), prefix, shared
         self.router = Linear(hidden, n_experts, prefix + "router")
         self.router_bias = self.w_gate_up = self.w_down = None
+        self.for_products = None      # per expert (gate and up, down) as the matrix products take them
 
     def tensor_specs(self):
         specs = self.router.tensor_specs() + [TensorSpec(self.prefix + "router.b", (self.n_experts,), "linear")]
@@ -96,13 +103,21 @@ class RoutedExperts:
             self.shared.load(get)
 
     def prepare(self, kernels):
+        """The stacked matrices stay row after row (the kernels for steps of few rows read them so).  For prompts every expert's
+        matrices are kept a second time in the kernel library's own form, where it has one for them: its products of many rows
+        read that form several times as fast, and a GPU with hundreds of GB holds both."""
         self.router.prepare(kernels)
         if self.shared is not None:
             self.shared.prepare(kernels)
+        if self.PACK_FOR_PROMPTS and hasattr(kernels, "pack_weight"):
+            self.for_products = [(kernels.pack_weight(self.w_gate_up[e]), kernels.pack_weight(self.w_down[e])) for e in range(self.n_experts)]
 
     def working_bytes(self, step) -> int:
         total = self.router.working_bytes(step, step.rows, out_size=4) + 2 * step.matrix(step.rows, self.top, 4)
-        total += step.matrix(step.rows * self.top, self.ff)
+        pairs = step.rows * self.top
+        total += step.matrix(self.n_experts, step.rows, 4) + step.matrix(pairs, self.ff) + step.matrix(pairs, self.hidden, 4)
+        if step.rows > step.seqs and pairs >= self.PRODUCT_PAIRS * self.n_experts:      # a step of many rows: the pairs' inputs, gate and up
+            total += step.matrix(pairs, self.hidden) + step.matrix(pairs, 2 * self.ff) + step.matrix(pairs, 1, 4)
         return total + (self.shared.working_bytes(step) if self.shared is not None else 0)
 
     def forward(self, ctx, x, hidden, then_norm=None):
@@ -113,12 +128,54 @@ class RoutedExperts:
         weights = ctx.new_f32(n, self.top)
         k.route_top_k(logits, self.router_bias, chosen, weights)
         ctx.extras["routing"] = (chosen, weights)
-        inner = ctx.new_activations(n * self.top, self.ff)
-        k.experts_gate_up(x, chosen, self.w_gate_up, inner, self.limit, self.alpha)
-        k.experts_down(inner, chosen, weights, self.w_down, hidden)
+        pairs = n * self.top
+        takes = getattr(k, "experts_rows_take", None)
+        if takes is None or not (takes(self.hidden) and takes(self.ff)):
+            inner = ctx.new_activations(pairs, self.ff)
+            k.experts_gate_up(x, chosen, self.w_gate_up, inner, self.limit, self.alpha)
+            k.experts_down(inner, chosen, weights, self.w_down, hidden)
+        else:
+            lists = torch.empty((self.n_experts, n), dtype=torch.int32, device=ctx.device)
+            counts = torch.empty((self.n_experts,), dtype=torch.int32, device=ctx.device)
+            k.experts_group(chosen, lists, counts)
+            if ctx.is_decode or pairs < self.PRODUCT_PAIRS * self.n_experts:
+                inner = ctx.new_activations(pairs, self.ff)
+                k.experts_rows(x, self.top, lists, counts, self.w_gate_up, inner, gated=True, limit=self.limit, alpha=self.alpha)
+                y = ctx.new_f32(pairs, self.hidden)
+                k.experts_rows(inner, 1, lists, counts, self.w_down, y)
+                k.experts_combine(y, None, weights, hidden)
+            else:
+                self._as_products(ctx, x, lists, counts, weights, hidden)
         if self.shared is not None:
             self.shared.forward(ctx, x, hidden)
         return None
+
+
+    def _as_products(self, ctx, x, lists, counts, weights, hidden):
+        """Every expert's pairs as one stretch of rows through the framework's matrix products."""
+        k = ctx.kernels
+        n, pairs = x.shape[0], x.shape[0] * self.top
+        matrices = self.for_products or [(self.w_gate_up[e], self.w_down[e]) for e in range(self.n_experts)]
+        held = counts.cpu().tolist()              # the host waits for the routing here
+        starts, at = [], 0
+        for count in held:
+            starts.append(at)
+            at += count
+        offsets = torch.tensor(starts, dtype=torch.int32, device=ctx.device)
+        gathered = ctx.new_activations(pairs, self.hidden)
+        place = torch.empty((pairs,), dtype=torch.int32, device=ctx.device)
+        k.experts_gather(x, self.top, lists, counts, offsets, gathered, place)
+        both = ctx.new_activations(pairs, 2 * self.ff)
+        for e, (first, count) in enumerate(zip(starts, held)):
+            if count:
+                k.gemm(gathered[first:first + count], matrices[e][0], both[first:first + count])
+        inner = ctx.new_activations(pairs, self.ff)
+        k.clamped_glu(both, inner, self.limit, self.alpha)
+        y = ctx.new_f32(pairs, self.hidden)
+        for e, (first, count) in enumerate(zip(starts, held)):
+            if count:
+                k.gemm(inner[first:first + count], matrices[e][1], y[first:first + count])
+        k.experts_combine(y, place, weights, hidden)
 
 
 @FEED_FORWARDS.register("routed_experts")

@@ -68,7 +68,10 @@ class StateSpaceScan:
         return CacheNeed(kind="state", state_shape=(self.state_floats + (self.taps - 1) * self.conv_width,), state_dtype=torch.float32)
 
     def working_bytes(self, step) -> int:
-        return (self.proj.working_bytes(step, step.rows) + step.matrix(step.rows, self.conv_width, 4) + step.matrix(step.rows, self.inner, 4)
+        chunks = 0
+        if step.sizes is not None and hasattr(step.sizes, "ssm_chunk_bytes"):
+            chunks = step.sizes.ssm_chunk_bytes(step.seqs, step.rows, step.max_rows_per_seq, self.n_heads, self.vdim, self.n_state)
+        return (chunks + self.proj.working_bytes(step, step.rows) + step.matrix(step.rows, self.conv_width, 4) + step.matrix(step.rows, self.inner, 4)
                 + step.matrix(step.rows, self.inner, reader=self.out.reader_for_plan(step.act_size))
                 + self.out.working_bytes(step, step.rows, accumulate=True))
 
@@ -83,7 +86,7 @@ class StateSpaceScan:
             k.short_conv_state(proj, self.inner, self.conv_width, self.taps, cache.state, self.state_floats, ctx.seq_start, ctx.seq_slot)
         y = ctx.new_f32(n, self.inner)
         k.ssm_scan(xbc, proj, self.dt_first, self.dt_bias, self.a_log, self.d_skip, cache.state, 0, ctx.seq_start, ctx.seq_slot, y,
-                   self.n_heads, self.vdim, self.n_state, self.n_groups)
+                   self.n_heads, self.vdim, self.n_state, self.n_groups, max_rows_per_seq=ctx.max_rows_per_seq)
         normed = ctx.new_activations(n, self.inner, reader=self.out.reader())
         k.gated_group_rmsnorm(y, proj, 0, self.norm_weight, self.norm_eps, normed, self.norm_groups)
         self.out.forward(ctx, normed, out=hidden, accumulate=True)

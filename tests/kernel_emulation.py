@@ -308,7 +308,7 @@ class TorchKernels:
 
     # ---- a state-space recurrence ----
     def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
-                 n_state, n_groups):
+                 n_state, n_groups, max_rows_per_seq=None):
         self.calls.append("ssm_scan")
         inner, per = n_heads * vdim, n_heads // n_groups
         region = self._region(state, state_offset, n_heads * n_state * vdim)
@@ -362,6 +362,40 @@ class TorchKernels:
             for j in range(top):
                 total += float(weights[row, j]) * (w_down[int(chosen[row, j])].double() @ inner[row * top + j].double())
             hidden[row] += total.float()
+
+    def experts_group(self, chosen, lists, counts):
+        self.calls.append("experts_group")
+        flat = chosen.reshape(-1)
+        for e in range(counts.shape[0]):
+            found = torch.nonzero(flat == e).reshape(-1).to(torch.int32)
+            counts[e] = found.numel()
+            lists[e, :found.numel()] = found
+
+    def experts_rows_take(self, inputs):
+        return inputs % 8 == 0
+
+    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0):
+        self.calls.append("experts_rows")
+        for e in range(counts.shape[0]):
+            for pair in lists[e, :int(counts[e])].tolist():
+                result = w[e].double() @ rows[pair // rows_per_pair_row].double()
+                if gated:
+                    half = result.shape[0] // 2
+                    result = self._clamped_glu(result[:half], result[half:], limit, alpha)
+                out[pair] = result.to(out.dtype)
+
+    def experts_gather(self, x, top, lists, counts, offsets, gathered, place):
+        self.calls.append("experts_gather")
+        for e in range(counts.shape[0]):
+            for i, pair in enumerate(lists[e, :int(counts[e])].tolist()):
+                gathered[int(offsets[e]) + i] = x[pair // top]
+                place[pair] = int(offsets[e]) + i
+
+    def experts_combine(self, y, place, weights, hidden):
+        self.calls.append("experts_combine")
+        n, top = weights.shape
+        index = (place if place is not None else torch.arange(n * top)).long().reshape(n, top)
+        hidden.add_((weights.double()[:, :, None] * y.double()[index]).sum(1).float())
 
     def clamped_glu(self, gate_up, out, limit, alpha):
         self.calls.append("clamped_glu")
