@@ -468,12 +468,11 @@ def pudorax_kernels(K, torch, width, heads, context, experts=32, top=4):
         wq, wk = torch.ones(q_w, device=dev), torch.ones(k_w, device=dev)
 
         def convolved_write():
-            K.short_conv(proj, 0, conv_weight, None, conv_state, 0, row_seq, starts, slots, conv)
+            K.conv_norm_rope_write(proj, 0, conv_weight, conv_state, 0, starts, slots, wq, wk, 1e-6, freq, 64, positions, row_seq, q_out,
+                                   k_pages, v_pages, table, heads, kv_heads, dim, vdim, dim, True)
             K.short_conv_state(proj, 0, conv_w, taps, conv_state, 0, starts, slots)
-            K.whole_norm_rope_write(conv, wq, wk, 1e-6, freq, 64, positions, row_seq, q_out, k_pages, v_pages, table, heads, kv_heads,
-                                    dim, vdim, dim, True)
         us = timed(convolved_write, torch)
-        note(f"short_conv + state + whole_norm_rope_write, {tag}", us, 2 * rows * conv_w * 2)
+        note(f"conv_norm_rope_write + short_conv_state, {tag}", us, 2 * rows * conv_w * 2)
         head_weight = torch.ones(dim, device=dev)
         cos = torch.ones(past + each, dim // 2, device=dev)
         qkv = torch.randn(rows, conv_w, device=dev).to(bf16)

@@ -379,20 +379,20 @@ extern "C" int bh_experts_gather(const void* x, int dtype, int top, const int32_
 // y [*][D] float32: the result of pair p lies at row place[p] (or p where no places are given).
 __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ place,
                                                               const float* __restrict__ weights, float* __restrict__ hidden, int top, int D) {
-  const int row = blockIdx.x;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float total = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const int pair = row * top + j;
-      total = fmaf(weights[pair], y[(size_t)(place ? place[pair] : pair) * D + d], total);
-    }
-    hidden[(size_t)row * D + d] += total;
+  const int row = blockIdx.x, d = blockIdx.y * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int pair = row * top + j;
+    total = fmaf(weights[pair], y[(size_t)(place ? place[pair] : pair) * D + d], total);
   }
+  hidden[(size_t)row * D + d] += total;
 }
 
 extern "C" int bh_experts_combine(const float* y, const int32_t* place, const float* weights, float* hidden, int n_rows, int top, int D,
                                   hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && top > 0 && D > 0, "experts_combine: sizes must be positive");
-  experts_combine_kernel<<<n_rows, 256, 0, stream>>>(y, place, weights, hidden, top, D);
+  BH_REQUIRE((D + 255) / 256 <= 65535, "experts_combine: rows of up to 16 million outputs");
+  experts_combine_kernel<<<dim3(n_rows, (D + 255) / 256), 256, 0, stream>>>(y, place, weights, hidden, top, D);
   return bh_check_launch("experts_combine");
 }

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const float* __restrict_
                                                         const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
                                                         float* __restrict__ y, int H, int vdim, int N, int G, int slices, int chunk_rows,
                                                         int chunks_per_seq) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   float* bc = lds;                                 // [SS_STAGE][2 N]: B, C of a row
   float* xs = bc + SS_STAGE * 2 * N;               // [SS_STAGE][vdim]
   float* part = xs + SS_STAGE * vdim;              // [SS_STAGE][slices][vdim]
@@ -141,14 +141,31 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const float* __restrict_
   for (int i = 0; i < NPT; ++i) S[i] = (MODE != 1 && works && n0 + i < n1) ? home[(size_t)(n0 + i) * vdim + p] : 0.f;
   const float rate = expf(a_log[head]), skip = d_skip[head], bias = dt_bias[head];
   float run = 0.f;
+  const int staged = 2 * N + vdim;      // a row's B, C and x, as they are asked for: eight loads a thread in flight
+  const bool by_four = per % 4 == 0 && N % 4 == 0;
   for (int r0 = start; r0 < stop; r0 += SS_STAGE) {
     const int rows = stop - r0 < SS_STAGE ? stop - r0 : SS_STAGE;
-    for (int e = threadIdx.x; e < rows * 2 * N; e += blockDim.x) {
-      const int r = e / (2 * N), j = e % (2 * N);
-      bc[r * 2 * N + j] = xbc[(size_t)(r0 + r) * xbc_stride + inner + (j < N ? group * N + j : (G + group) * N + j - N)];
+    for (int e0 = threadIdx.x; e0 < rows * staged; e0 += 8 * blockDim.x) {
+      float got[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = e0 + u * blockDim.x;
+        if (e < rows * staged) {
+          const int r = e / staged, j = e % staged;
+          const int column = j < N ? inner + group * N + j : (j < 2 * N ? inner + (G + group) * N + j - N : head * vdim + j - 2 * N);
+          got[u] = xbc[(size_t)(r0 + r) * xbc_stride + column];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = e0 + u * blockDim.x;
+        if (e < rows * staged) {
+          const int r = e / staged, j = e % staged;
+          if (j < 2 * N) bc[r * 2 * N + j] = got[u];
+          else xs[r * vdim + j - 2 * N] = got[u];
+        }
+      }
     }
-    for (int e = threadIdx.x; e < rows * vdim; e += blockDim.x)
-      xs[e] = xbc[(size_t)(r0 + e / vdim) * xbc_stride + head * vdim + e % vdim];
     if (threadIdx.x < rows) {
       if (MODE == 2) {
         fac[2 * threadIdx.x] = expf(cum[(size_t)(r0 + threadIdx.x) * H + head]);
@@ -170,16 +187,30 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const float* __restrict_
         const float* b = bc + r * 2 * N;
         const float* c = b + N;
         float acc = 0.f;
-        if (MODE == 2) {
+        const float decay = MODE == 2 ? 0.f : expf(fac[2 * r]), dtx = MODE == 2 ? 0.f : fac[2 * r + 1] * xs[r * vdim + p];
+        if (by_four) {      // four state rows a read of LDS
 #pragma unroll
-          for (int i = 0; i < NPT; ++i)
-            if (n0 + i < n1) acc = fmaf(S[i], c[n0 + i], acc);
+          for (int i = 0; i < NPT; i += 4) {
+            if (n0 + i < n1) {
+              const float4 c4 = *reinterpret_cast<const float4*>(c + n0 + i);
+              if (MODE != 2) {
+                const float4 b4 = *reinterpret_cast<const float4*>(b + n0 + i);
+                S[i] = fmaf(decay, S[i], b4.x * dtx);
+                S[i + 1] = fmaf(decay, S[i + 1], b4.y * dtx);
+                S[i + 2] = fmaf(decay, S[i + 2], b4.z * dtx);
+                S[i + 3] = fmaf(decay, S[i + 3], b4.w * dtx);
+              }
+              acc = fmaf(S[i], c4.x, acc);
+              acc = fmaf(S[i + 1], c4.y, acc);
+              acc = fmaf(S[i + 2], c4.z, acc);
+              acc = fmaf(S[i + 3], c4.w, acc);
+            }
+          }
         } else {
-          const float decay = expf(fac[2 * r]), dtx = fac[2 * r + 1] * xs[r * vdim + p];
 #pragma unroll
           for (int i = 0; i < NPT; ++i) {
             if (n0 + i < n1) {
-              S[i] = fmaf(decay, S[i], b[n0 + i] * dtx);
+              if (MODE != 2) S[i] = fmaf(decay, S[i], b[n0 + i] * dtx);
               acc = fmaf(S[i], c[n0 + i], acc);
             }
           }

@@ -97,19 +97,26 @@ extern "C" int bh_whole_norm_rope_write(const float* qkv, const float* wq, const
 // its state) is made on the way, a row's convolved channels stand in LDS as float32 and are never written to memory.
 // proj [n_rows][row_stride]: a row holds, from `first`, q, k and v; w_conv [q + k + v channels][taps] (taps 0: no convolution).
 template <typename T>
-__global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
+__global__ __launch_bounds__(1024) void conv_norm_rope_write_kernel(
     const T* __restrict__ proj, int row_stride, int first, const float* __restrict__ w_conv, int taps, const float* __restrict__ state,
     long slot_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write) {
-  extern __shared__ float conv[];      // [q | k | v] of this row
-  __shared__ float scratch[8];
+  extern __shared__ float conv[];      // [q | k | v] of this row, then the cosines and sines of the row's turned pairs
+  __shared__ float scratch[16];
   const int row = blockIdx.x;
   const int q_width = H * dim, k_width = G * dim, v_width = G * vdim, channels = q_width + k_width + v_width;
+  float* cosines = conv + channels;
+  float* sines = cosines + turned / 2;
   const int seq = row_seq[row], pos = positions[row];
   const int t = row - seq_start[seq];
   const float* old = state ? state + (size_t)seq_slot[seq] * slot_stride : nullptr;
+  for (int i = threadIdx.x; i < turned / 2; i += blockDim.x) {
+    const float angle = (float)pos * freq[i];
+    cosines[i] = cosf(angle);
+    sines[i] = sinf(angle);
+  }
   float ss_q = 0.f, ss_k = 0.f;
   for (int c = threadIdx.x; c < channels; c += blockDim.x) {
     float acc;
@@ -142,8 +149,7 @@ __global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
       if (i < turned) {
         const int mate = at ^ 1;
         const float other = q[mate] * inv_q * wq[mate];
-        const float angle = (float)pos * freq[i >> 1];
-        const float c = cosf(angle), s = sinf(angle);
+        const float c = cosines[i >> 1], s = sines[i >> 1];
         y = (i & 1) ? y * c + other * s : y * c - other * s;
       }
     }
@@ -160,8 +166,7 @@ __global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
       if (i < turned) {
         const int mate = at ^ 1;
         const float other = k[mate] * inv_k * wk[mate];
-        const float angle = (float)pos * freq[i >> 1];
-        const float c = cosf(angle), s = sinf(angle);
+        const float c = cosines[i >> 1], s = sines[i >> 1];
         y = (i & 1) ? y * c + other * s : y * c - other * s;
       }
     }
@@ -188,13 +193,14 @@ extern "C" int bh_conv_norm_rope_write(const void* proj, int dtype, int row_stri
   BH_REQUIRE(first >= 0 && first + channels <= row_stride, "conv_norm_rope_write: q, k and v lie outside a row of %d", row_stride);
   BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && pad % 32 == 0),
              "conv_norm_rope_write: cache order %d does not exist for head size %d", kv_order, pad);
-  const size_t lds = (size_t)channels * sizeof(float);
+  const size_t lds = (size_t)(channels + turned) * sizeof(float);
   BH_REQUIRE(lds <= 128 * 1024, "conv_norm_rope_write: %d channels do not fit the local memory", channels);
+  const int threads = n_rows < 2 * bh_compute_units() && channels >= 2048 ? 1024 : 256;      // few rows: more of the chip a row
 #define BH_CW(T)                                                                                                                   \
   do {                                                                                                                             \
     if (lds > 48 * 1024)                                                                                                           \
       (void)hipFuncSetAttribute((const void*)conv_norm_rope_write_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-    conv_norm_rope_write_kernel<T><<<n_rows, 256, lds, stream>>>((const T*)proj, row_stride, first, w_conv, taps, state, slot_stride,  \
+    conv_norm_rope_write_kernel<T><<<n_rows, threads, lds, stream>>>((const T*)proj, row_stride, first, w_conv, taps, state, slot_stride,  \
                                                                  seq_start, seq_slot, wq, wk, eps, freq, turned, positions, row_seq, \
                                                                  (T*)q_out, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, G, \
                                                                  dim, vdim, pad, kv_order, write);                                  \
