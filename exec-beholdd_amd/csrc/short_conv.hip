@@ -41,6 +41,50 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const T* __restrict__ u
   }
 }
 
+// The same for steps of many rows: a thread walks SC_ROWS consecutive rows of its channel with the last TAPS inputs in
+// registers, so that every input is loaded once (where a sequence starts inside the stretch, the window is filled anew
+// from that sequence's state).
+#define SC_ROWS 32
+
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void short_conv_walk_kernel(const T* __restrict__ u, int row_stride, int first,
+                                                              const float* __restrict__ w, const float* __restrict__ bias,
+                                                              const float* __restrict__ state, long slot_stride,
+                                                              const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_start,
+                                                              const int32_t* __restrict__ seq_slot, float* __restrict__ out,
+                                                              int n_rows, int channels, int silu) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  float wc[TAPS], win[TAPS];
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) wc[j] = w[(size_t)c * TAPS + j];
+  const float b = bias ? bias[c] : 0.f;
+  const int r0 = blockIdx.y * SC_ROWS, r1 = r0 + SC_ROWS < n_rows ? r0 + SC_ROWS : n_rows;
+  int seq = -1;
+  for (int row = r0; row < r1; ++row) {
+    const int here = row_seq[row];
+    if (here != seq) {      // the first row of the stretch, or of a sequence: the inputs before it
+      seq = here;
+      const int t = row - seq_start[seq];
+      const float* old = state + (size_t)seq_slot[seq] * slot_stride;
+#pragma unroll
+      for (int j = 0; j < TAPS - 1; ++j) {
+        const int back = TAPS - 1 - j;
+        win[j] = back <= t ? to_f32(u[(size_t)(row - back) * row_stride + first + c]) : old[(size_t)(TAPS - 1 + t - back) * channels + c];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TAPS - 1; ++j) win[j] = win[j + 1];
+    }
+    win[TAPS - 1] = to_f32(u[(size_t)row * row_stride + first + c]);
+    float acc = b;
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) acc = fmaf(wc[j], win[j], acc);
+    if (silu) acc = acc / (1.0f + expf(-acc));
+    out[(size_t)row * channels + c] = acc;
+  }
+}
+
 extern "C" int bh_short_conv(const void* u, int dtype, int row_stride, int first, const float* w, const float* bias,
                              const float* state, long slot_stride, const int32_t* row_seq, const int32_t* seq_start,
                              const int32_t* seq_slot, float* out, int n_rows, int channels, int taps, int silu,
@@ -50,6 +94,23 @@ extern "C" int bh_short_conv(const void* u, int dtype, int row_stride, int first
   BH_REQUIRE(first >= 0 && first + channels <= row_stride, "short_conv: channels %d..%d lie outside a row of %d", first,
              first + channels, row_stride);
   BH_REQUIRE(taps == 1 || state != nullptr, "short_conv: more than one tap needs a state");
+  if (n_rows >= 4 * SC_ROWS && taps >= 2 && taps <= 4 && (dtype == BH_F32 || dtype == BH_BF16)) {
+    dim3 walk((channels + 255) / 256, (n_rows + SC_ROWS - 1) / SC_ROWS);
+#define BH_SW(T, TAPS)                                                                                                              \
+  short_conv_walk_kernel<T, TAPS><<<walk, 256, 0, stream>>>((const T*)u, row_stride, first, w, bias, state, slot_stride, row_seq, seq_start, \
+                                                            seq_slot, out, n_rows, channels, silu)
+    if (dtype == BH_F32) {
+      if (taps == 2) BH_SW(float, 2);
+      else if (taps == 3) BH_SW(float, 3);
+      else BH_SW(float, 4);
+    } else {
+      if (taps == 2) BH_SW(bf16_t, 2);
+      else if (taps == 3) BH_SW(bf16_t, 3);
+      else BH_SW(bf16_t, 4);
+    }
+#undef BH_SW
+    return bh_check_launch("short_conv");
+  }
   dim3 grid((channels + 255) / 256, n_rows < 4096 ? n_rows : 4096);
   if (dtype == BH_F32)
     short_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, row_stride, first, w, bias, state, slot_stride, row_seq,

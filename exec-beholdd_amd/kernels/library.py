@@ -252,6 +252,17 @@ class KernelSizes:
                     int(self.lib.bh_sample_top_k_scratch(int(n_rows), int(vocab))))
         return _rounded(words * 4) + 4 * _rounded(n_rows * 4)
 
+    def ssm_chunk_bytes(self, n_seqs, n_rows, max_rows, n_heads, vdim, n_state) -> int:
+        """Bytes of scratch memory that `ssm_scan` allocates for a step of these sizes (sequences cut into chunks)."""
+        if not self.lib.bh_ssm_fast_takes(int(vdim), int(n_state)):
+            return 0
+        chunk_rows = int(self.lib.bh_ssm_chunk_rows(int(n_seqs), int(max_rows), int(n_heads)))
+        chunks = -(-int(max_rows) // chunk_rows)
+        if chunks <= 1:
+            return 0
+        return (_rounded(n_seqs * chunks * n_heads * n_state * vdim * 4) + _rounded(n_seqs * chunks * n_heads * 4)
+                + _rounded(n_rows * n_heads * 4))
+
     def packs(self, rows, cols, act_size) -> bool:
         """Whether `pack_weight` regroups a matrix of this shape and element size."""
         return act_size == 2 and cols % 64 == 0
@@ -1054,12 +1065,21 @@ class HipKernels(KernelSizes):
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
             self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
 
+    CONV_WALK_ROWS = 128      # from that many rows a step's convolution walks down the rows (csrc/short_conv.hip)
+
     def conv_norm_rope_write(self, proj, first, conv_weight, state, state_offset, seq_start, seq_slot, q_weight, k_weight, eps, freq,
                              turned, positions, row_seq, q_out, k_pages, v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
         """`short_conv` of the q, k, v channels of `proj` (from column `first`; conv_weight f32 [channels, taps], or None for no
         convolution) and `whole_norm_rope_write` of the result in one launch: the convolved row is never written to memory.  The
-        state is read, not updated (`short_conv_state` afterwards)."""
+        state is read, not updated (`short_conv_state` afterwards).  A step of many rows runs the two kernels after all: the
+        convolution that walks down the rows loads every input once, where a workgroup per row loads it once per tap."""
         n_rows = proj.shape[0]
+        if n_rows >= self.CONV_WALK_ROWS and conv_weight is not None and 2 <= conv_weight.shape[1] <= 4:
+            conv = torch.empty((n_rows, conv_weight.shape[0]), dtype=torch.float32, device=self.device)
+            self.short_conv(proj, first, conv_weight, None, state, state_offset, row_seq, seq_start, seq_slot, conv)
+            self.whole_norm_rope_write(conv, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages, v_pages, page_table,
+                                       n_heads, n_kv_heads, dim, vdim, pad, write_kv)
+            return
         channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
         taps = conv_weight.shape[1] if conv_weight is not None else 0
         if tuple(q_out.shape) != (n_rows, n_heads * pad) or q_out.dtype != proj.dtype or (conv_weight is not None and conv_weight.shape[0] != channels):
@@ -1095,17 +1115,6 @@ class HipKernels(KernelSizes):
             gate.shape[1], int(gate_first), self._ptr(out, "gate_heads out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
 
     # ---- a state-space recurrence with a scalar decay per head ----
-    def ssm_chunk_bytes(self, n_seqs, n_rows, max_rows, n_heads, vdim, n_state) -> int:
-        """Bytes of scratch memory that `ssm_scan` allocates for a step of these sizes (sequences cut into chunks)."""
-        if not self.lib.bh_ssm_fast_takes(int(vdim), int(n_state)):
-            return 0
-        chunk_rows = int(self.lib.bh_ssm_chunk_rows(int(n_seqs), int(max_rows), int(n_heads)))
-        chunks = -(-int(max_rows) // chunk_rows)
-        if chunks <= 1:
-            return 0
-        return (_rounded(n_seqs * chunks * n_heads * n_state * vdim * 4) + _rounded(n_seqs * chunks * n_heads * 4)
-                + _rounded(n_rows * n_heads * 4))
-
     def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
                  n_state, n_groups, max_rows_per_seq=None):
         """Per (sequence, head): S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x with dt = softplus(proj[:, dt_first

@@ -109,7 +109,9 @@ def test_small_row_kernels(K, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channels,taps,lengths,silu", [(70, 4, [5, 1, 31], True), (300, 2, [1, 1, 1], False), (33, 5, [2, 3, 1, 40], True),
-                                                        (8, 1, [4, 9], False), (520, 3, [130], True)])
+                                                        (8, 1, [4, 9], False), (520, 3, [130], True),
+                                                        (70, 4, [100, 3, 60, 1, 40], True),      # many rows: the walk down the rows, sequences starting inside a stretch
+                                                        (300, 2, [33, 31, 64, 1, 1, 70], False)])
 def test_short_conv_and_its_state(K, dtype, channels, taps, lengths, silu):
     """A step's rows after a past of the same length: the state left by the past's step is what the present's rows read,
     also where a sequence brings fewer rows than the state holds."""
