@@ -581,10 +581,11 @@ def pudorax_expert_calls(K, torch, x, chosen, shares, w_gu, w_d, hidden, active,
         return
     part = RoutedExperts(width, experts, top, ff, 7.0, "m.")
     part.w_gate_up, part.w_down = w_gu, w_d
-    part.for_products = [(K.pack_weight(w_gu[e]), K.pack_weight(w_d[e])) for e in range(experts)]
+    part.prepare(K)
     ctx = SimpleNamespace(kernels=K, device=x.device, new_f32=lambda *shape: torch.empty(shape, device=x.device),
                           new_activations=lambda *shape, reader=None: torch.empty(shape, device=x.device, dtype=x.dtype))
-    yield (f"experts as products (gather, {2 * experts} products, clamped_glu, combine)", lambda: part._as_products(ctx, x, lists, counts, shares, hidden),
+    form = "two launches over all experts" if part.in_one_launch else f"{2 * experts} products, clamped_glu"
+    yield (f"experts of a prompt (gather, {form}, combine)", lambda: part._as_products(ctx, x, lists, counts, shares, hidden),
            weights_read + pairs * (2 * width + 3 * ff) * 2 + pairs * width * 8, 6.0 * pairs * ff * width)
 
 

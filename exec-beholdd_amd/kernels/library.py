@@ -192,6 +192,8 @@ class KernelSizes:
             "bh_ssm_scan_fast": [p, i, p, i, i, i, p, p, p, p, ctypes.c_long, p, p, p, p, p, p, i, i, i, i, i, i, i, p],
             "bh_ssm_chunk_rows": [i, i, i],
             "bh_ssm_fast_takes": [i, i],
+            "bh_experts_products": [p, p, p, i, p, i, i, i, f, f, p],
+            "bh_experts_products_takes": [i, i],
             "bh_experts_group": [p, i, p, i, p, i, p],
             "bh_experts_rows": [p, i, i, p, i, p, p, p, i, i, i, i, f, f, p],
             "bh_experts_gather": [p, i, i, p, i, p, p, p, p, i, i, i, p],
@@ -1225,6 +1227,24 @@ class HipKernels(KernelSizes):
             self._ptr(rows, "experts rows"), _code(rows, "experts rows"), int(rows_per_pair_row), self._ptr(lists, "lists", (torch.int32,)),
             lists.shape[1], self._ptr(counts, "counts", (torch.int32,)), self._ptr(w, "expert weights"), self._ptr(out, "experts out"),
             experts, k, n, int(bool(gated)), float(limit), float(alpha), self._stream()))
+
+    def experts_products_take(self, dtype, inputs: int, outputs: int) -> bool:
+        """Whether `experts_products` takes products of these sizes and element type."""
+        return dtype == torch.bfloat16 and bool(self.lib.bh_experts_products_takes(int(inputs), int(outputs)))
+
+    def experts_products(self, rows, w, tiles, out, gated=False, limit=0.0, alpha=0.0):
+        """All experts' products of a prompt in one launch on the matrix cores: rows bf16 [pairs, K] lie expert after expert,
+        tiles int32 [n, 3] = (expert, first row, rows of the tile: 1 to 128) names every stretch; gated: w [E, 2 N, K] and out
+        bf16 [pairs, N] = act(gate, up); otherwise w [E, N, K] and out float32 [pairs, N]."""
+        experts, w_rows, k = w.shape
+        n = w_rows // 2 if gated else w_rows
+        if rows.shape[1] != k or tuple(out.shape) != (rows.shape[0], n) or rows.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 \
+                or out.dtype != (torch.bfloat16 if gated else torch.float32) or tiles.dim() != 2 or tiles.shape[1] != 3:
+            raise KernelError(f"experts_products: shapes rows {tuple(rows.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_experts_products(
+            self._ptr(rows, "experts rows", (torch.bfloat16,)), self._ptr(w, "expert weights", (torch.bfloat16,)),
+            self._ptr(tiles, "tiles", (torch.int32,)), tiles.shape[0], self._ptr(out, "experts out"), k, n, int(bool(gated)), float(limit),
+            float(alpha), self._stream()))
 
     def experts_gather(self, x, top, lists, counts, offsets, gathered, place):
         """gathered[offsets[e] + i] = x[lists[e, i] // top] and place[lists[e, i]] = offsets[e] + i for i < counts[e]: the pairs'

@@ -10,7 +10,9 @@ all.  The (row, choice) pairs are grouped by expert on the device (`experts_grou
 workgroup per expert and block of outputs that reads the expert's rows from memory once for all of its pairs
 (`experts_rows`), with nothing that depends on the routing on the host, so that decode steps can be captured.  A step
 of many rows (a prompt) reads the experts' counts on the host (the step waits for the device there), lays the pairs'
-inputs side by side, expert after expert, and runs the framework's matrix products on each expert's stretch.  Sizes
+inputs side by side, expert after expert, and runs all experts' products in one launch on the matrix cores
+(`experts_products`, over a table of row tiles made from the counts; the activation rides in the first product), or,
+for sizes and element types that kernel does not take, the framework's matrix products on each expert's stretch.  Sizes
 that the grouped kernels do not take go pair by pair (`experts_gate_up`, `experts_down`).  In every form a row's
 experts' shares are added in the order of its own choice, so its result depends on its batch-mates by rounding at most.  The routing is left in
 `ctx.extras["routing"]` ((chosen, weights) of the last layer that ran).  Every size and constant is a constructor
@@ -80,6 +82,7 @@ class RoutedExperts:
         self.router = Linear(hidden, n_experts, prefix + "router")
         self.router_bias = self.w_gate_up = self.w_down = None
         self.for_products = None      # per expert (gate and up, down) as the matrix products take them
+        self.in_one_launch = False    # a prompt's products run as one launch over all experts (kernels.experts_products)
 
     def tensor_specs(self):
         specs = self.router.tensor_specs() + [TensorSpec(self.prefix + "router.b", (self.n_experts,), "linear")]
@@ -109,7 +112,9 @@ class RoutedExperts:
         self.router.prepare(kernels)
         if self.shared is not None:
             self.shared.prepare(kernels)
-        if self.PACK_FOR_PROMPTS and hasattr(kernels, "pack_weight"):
+        takes = getattr(kernels, "experts_products_take", None)
+        self.in_one_launch = bool(takes is not None and takes(self.w_gate_up.dtype, self.hidden, self.ff) and takes(self.w_down.dtype, self.ff, self.hidden))
+        if self.PACK_FOR_PROMPTS and hasattr(kernels, "pack_weight") and not self.in_one_launch:
             self.for_products = [(kernels.pack_weight(self.w_gate_up[e]), kernels.pack_weight(self.w_down[e])) for e in range(self.n_experts)]
 
     def working_bytes(self, step) -> int:
@@ -165,6 +170,15 @@ class RoutedExperts:
         gathered = ctx.new_activations(pairs, self.hidden)
         place = torch.empty((pairs,), dtype=torch.int32, device=ctx.device)
         k.experts_gather(x, self.top, lists, counts, offsets, gathered, place)
+        if self.in_one_launch:
+            tiles = torch.tensor([(e, first + at, min(128, count - at)) for e, (first, count) in enumerate(zip(starts, held))
+                                  for at in range(0, count, 128)], dtype=torch.int32, device=ctx.device)
+            inner = ctx.new_activations(pairs, self.ff)
+            k.experts_products(gathered, self.w_gate_up, tiles, inner, gated=True, limit=self.limit, alpha=self.alpha)
+            y = ctx.new_f32(pairs, self.hidden)
+            k.experts_products(inner, self.w_down, tiles, y)
+            k.experts_combine(y, place, weights, hidden)
+            return
         both = ctx.new_activations(pairs, 2 * self.ff)
         for e, (first, count) in enumerate(zip(starts, held)):
             if count:

@@ -318,6 +318,31 @@ def test_routed_experts_kernels(K, dtype, rows, width, experts, top, ff, limit):
     assert rel(out, g / (1 + np.exp(-1.702 * g)) * (u + 1)) < tol(dtype, bf16=8e-3)
 
 
+@pytest.mark.parametrize("inputs,outputs,counts", [(64, 40, [0, 5, 130, 128, 1, 257]), (128, 64, [3, 0, 0, 70]), (192, 200, [129, 127, 256]),
+                                                   (1024, 384, [300, 1, 60, 0, 515])])
+def test_all_experts_products_in_one_launch(K, inputs, outputs, counts):
+    """Stretches of rows that end at, before and after a tile's end, experts without rows, outputs that fill no whole block."""
+    rng = np.random.default_rng(inputs + outputs)
+    experts, total, limit = len(counts), sum(counts), 1.5
+    rows_t, rows = rounded(rng.standard_normal((total, inputs)), torch.bfloat16)
+    gate_up_t, gate_up = rounded(rng.standard_normal((experts, 2 * outputs, inputs)) / np.sqrt(inputs) * 2, torch.bfloat16)
+    plain_t, plain_w = rounded(rng.standard_normal((experts, outputs, inputs)) / np.sqrt(inputs), torch.bfloat16)
+    starts = np.concatenate([[0], np.cumsum(counts)])
+    tiles = dev(np.array([(e, starts[e] + at, min(128, c - at)) for e, c in enumerate(counts) for at in range(0, c, 128)], np.int32))
+    gated = torch.full((total, outputs), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    K.experts_products(dev(rows_t), dev(gate_up_t), tiles, gated, gated=True, limit=limit, alpha=1.702)
+    sums = torch.full((total, outputs), 7.0, device="cuda:0")
+    K.experts_products(dev(rows_t), dev(plain_t), tiles, sums)
+    for e, c in enumerate(counts):
+        if not c:
+            continue
+        x = rows[starts[e]:starts[e + 1]].astype(np.float64)
+        both = x @ gate_up[e].astype(np.float64).T
+        g, u = np.minimum(both[:, :outputs], limit), np.clip(both[:, outputs:], -limit, limit)
+        assert rel(gated[starts[e]:starts[e + 1]], g / (1 + np.exp(-1.702 * g)) * (u + 1)) < 1e-2, e
+        assert rel(sums[starts[e]:starts[e + 1]], x @ plain_w[e].astype(np.float64).T) < 2e-5, e
+
+
 # ---- the engine over every cut ------------------------------------------------------------------------------------
 
 @pytest.fixture(scope="module")
