@@ -584,7 +584,8 @@ def pudorax_expert_calls(K, torch, x, chosen, shares, w_gu, w_d, hidden, active,
     part.prepare(K)
     ctx = SimpleNamespace(kernels=K, device=x.device, new_f32=lambda *shape: torch.empty(shape, device=x.device),
                           new_activations=lambda *shape, reader=None: torch.empty(shape, device=x.device, dtype=x.dtype))
-    form = "two launches over all experts" if part.in_one_launch else f"{2 * experts} products, clamped_glu"
+    one = part.in_one_launch and 6.0 * pairs * ff * width <= part.ONE_LAUNCH_WORK
+    form = "two launches over all experts" if one else f"{2 * experts} products, clamped_glu"
     yield (f"experts of a prompt (gather, {form}, combine)", lambda: part._as_products(ctx, x, lists, counts, shares, hidden),
            weights_read + pairs * (2 * width + 3 * ff) * 2 + pairs * width * 8, 6.0 * pairs * ff * width)
 

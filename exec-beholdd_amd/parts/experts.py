@@ -72,6 +72,9 @@ class RoutedExperts:
     graph_safe_rows = 1       # steps of several rows a sequence may read the experts' counts on the host
     PRODUCT_PAIRS = 16        # from that many pairs an expert on average, a step of many rows runs matrix products
     PACK_FOR_PROMPTS = True   # keep a second copy of every expert's matrices in the form the products of many rows read fastest
+    ONE_LAUNCH_WORK = 1.5e11  # up to that many operations a layer, a prompt's experts run as one launch over all of them: the
+                              # one kernel reaches about 120 TFLOP/s whatever the size (tiles of 128 x 64 outputs re-read their
+                              # operands through the L2), the products per expert cost about 25 us each and then run faster
 
     def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared: ClampedGLU | None = None,
                  alpha: float = GATE_SLOPE):
@@ -114,7 +117,7 @@ class RoutedExperts:
             self.shared.prepare(kernels)
         takes = getattr(kernels, "experts_products_take", None)
         self.in_one_launch = bool(takes is not None and takes(self.w_gate_up.dtype, self.hidden, self.ff) and takes(self.w_down.dtype, self.ff, self.hidden))
-        if self.PACK_FOR_PROMPTS and hasattr(kernels, "pack_weight") and not self.in_one_launch:
+        if self.PACK_FOR_PROMPTS and hasattr(kernels, "pack_weight"):
             self.for_products = [(kernels.pack_weight(self.w_gate_up[e]), kernels.pack_weight(self.w_down[e])) for e in range(self.n_experts)]
 
     def working_bytes(self, step) -> int:
@@ -170,7 +173,7 @@ class RoutedExperts:
         gathered = ctx.new_activations(pairs, self.hidden)
         place = torch.empty((pairs,), dtype=torch.int32, device=ctx.device)
         k.experts_gather(x, self.top, lists, counts, offsets, gathered, place)
-        if self.in_one_launch:
+        if self.in_one_launch and 6.0 * pairs * self.ff * self.hidden <= self.ONE_LAUNCH_WORK:
             tiles = torch.tensor([(e, first + at, min(128, count - at)) for e, (first, count) in enumerate(zip(starts, held))
                                   for at in range(0, count, 128)], dtype=torch.int32, device=ctx.device)
             inner = ctx.new_activations(pairs, self.ff)
