@@ -71,6 +71,17 @@ int bh_check_launch(const char* what);
 // workgroups against.  Where no GPU is visible (a byte plan made on another machine) it says 256.
 int bh_compute_units();
 
+// Lets KERNEL use `bytes` of dynamic LDS where that is more than the 48 KB a kernel may use unasked.  The runtime is told
+// once per kernel and size (the first, eager run of a step): nothing is asked of it while a stream captures a graph.
+template <auto KERNEL>
+inline void bh_allow_lds(size_t bytes) {
+  static size_t allowed = 48 * 1024;
+  if (bytes > allowed) {
+    (void)hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    allowed = bytes;
+  }
+}
+
 #define BH_REQUIRE(cond, ...)                  \
   do {                                         \
     if (!(cond)) return bh_fail(__VA_ARGS__);  \

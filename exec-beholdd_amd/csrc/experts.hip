@@ -123,6 +123,8 @@ extern "C" int bh_experts_gate_up(const void* h, int dtype, const int32_t* chose
   BH_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, "experts_gate_up: rows of up to 16384 inputs, got %d", K);
   dim3 grid(n_rows * top, (ff + EX_OUTS - 1) / EX_OUTS);
   const size_t lds = (size_t)K * sizeof(float);
+  if (dtype == BH_F32) bh_allow_lds<experts_gate_up_kernel<float>>(lds);
+  if (dtype == BH_BF16) bh_allow_lds<experts_gate_up_kernel<bf16_t>>(lds);
   if (dtype == BH_F32)
     experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, lds, stream>>>((const float*)h, chosen, (const float*)w_gu, (float*)inner, top, K, ff,
                                                                        limit, alpha);
@@ -162,6 +164,8 @@ extern "C" int bh_experts_down(const void* inner, int dtype, const int32_t* chos
   const size_t lds = (size_t)top * ff * sizeof(float);
   BH_REQUIRE(lds <= 64 * 1024, "experts_down: %d experts a row of %d inner values do not fit the local memory", top, ff);
   dim3 grid(n_rows, (D + EX_OUTS - 1) / EX_OUTS);
+  if (dtype == BH_F32) bh_allow_lds<experts_down_kernel<float>>(lds);
+  if (dtype == BH_BF16) bh_allow_lds<experts_down_kernel<bf16_t>>(lds);
   if (dtype == BH_F32)
     experts_down_kernel<float><<<grid, 64 * EX_WAVES, lds, stream>>>((const float*)inner, chosen, weights, (const float*)w_d, hidden, top, ff, D);
   else if (dtype == BH_BF16)

@@ -82,13 +82,11 @@ extern "C" int bh_ssm_scan(const float* xbc, int xbc_stride, const void* proj, i
   BH_REQUIRE(lds_bytes <= 160 * 1024 - 64, "ssm_scan: a state of %d x %d does not fit the local memory", N, vdim);
   dim3 grid(n_seqs, H);
   if (dtype == BH_F32) {
-    if (lds_bytes > 48 * 1024)
-      (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    bh_allow_lds<ssm_scan_kernel<float>>(lds_bytes);
     ssm_scan_kernel<float><<<grid, 256, lds_bytes, stream>>>(xbc, xbc_stride, (const float*)proj, proj_stride, dt_first, dt_bias, a_log,
                                                              d_skip, state, slot_stride, seq_start, seq_slot, y, H, vdim, N, G, slices);
   } else if (dtype == BH_BF16) {
-    if (lds_bytes > 48 * 1024)
-      (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    bh_allow_lds<ssm_scan_kernel<bf16_t>>(lds_bytes);
     ssm_scan_kernel<bf16_t><<<grid, 256, lds_bytes, stream>>>(xbc, xbc_stride, (const bf16_t*)proj, proj_stride, dt_first, dt_bias,
                                                               a_log, d_skip, state, slot_stride, seq_start, seq_slot, y, H, vdim, N, G,
                                                               slices);
@@ -289,8 +287,7 @@ static int ssm_fast_launch(const float* xbc, int xbc_stride, const T* proj, int 
   dim3 grid(n_seqs * chunks_per_seq, H);
 #define BH_SS(MODE)                                                                                                                 \
   do {                                                                                                                              \
-    if (lds > 48 * 1024)                                                                                                            \
-      (void)hipFuncSetAttribute((const void*)ssm_chunk_kernel<T, NPT, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+    bh_allow_lds<ssm_chunk_kernel<T, NPT, MODE>>(lds);                                                                              \
     ssm_chunk_kernel<T, NPT, MODE><<<grid, 256, lds, stream>>>(xbc, xbc_stride, proj, proj_stride, dt_first, dt_bias, a_log, d_skip,   \
                                                                state, slot_stride, chunk_states, chunk_decay, cum, seq_start, seq_slot, \
                                                                y, H, vdim, N, G, slices, chunk_rows, chunks_per_seq);                \

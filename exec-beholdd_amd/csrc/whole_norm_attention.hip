@@ -198,8 +198,7 @@ extern "C" int bh_conv_norm_rope_write(const void* proj, int dtype, int row_stri
   const int threads = n_rows < 2 * bh_compute_units() && channels >= 2048 ? 1024 : 256;      // few rows: more of the chip a row
 #define BH_CW(T)                                                                                                                   \
   do {                                                                                                                             \
-    if (lds > 48 * 1024)                                                                                                           \
-      (void)hipFuncSetAttribute((const void*)conv_norm_rope_write_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    bh_allow_lds<conv_norm_rope_write_kernel<T>>(lds);                                                                             \
     conv_norm_rope_write_kernel<T><<<n_rows, threads, lds, stream>>>((const T*)proj, row_stride, first, w_conv, taps, state, slot_stride,  \
                                                                  seq_start, seq_slot, wq, wk, eps, freq, turned, positions, row_seq, \
                                                                  (T*)q_out, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, G, \

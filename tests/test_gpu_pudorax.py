@@ -574,6 +574,24 @@ def test_long_prompts_in_portions_and_long_decoding(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_tall_state_through_the_captured_steps(tmp_path, dtype):
+    """A state of 256 rows a head: the scan's stage needs more local memory than a kernel may use unasked, in the prompt's chunks
+    and in decode steps that are captured and replayed."""
+    config = {"architecture": "Pudorax", "vocab": 61, "width": 64, "norm": {"eps": 1e-5}, "token_side": {"dim": 8},
+              "layers": [pm.mamba2(2, 64, 256, 1, 2, 3, mlp=None), pm.attention(2, 1, 32, 32, 2, 0.2, 8, mlp=None)]}
+    weights = pm.random_weights(config, 13)
+    folder = pm.write_model(tmp_path / "tall", config, weights)
+    request = schedules.random_requests(config["vocab"], [300], seed=5)[0]
+    want = [plain.forward(config, weights, request)]
+    engine = engine_for(folder, dtype, max_tokens=512)
+    tolerances = tolerances_for(folder, dtype, [request], want, least=1e-4 if dtype == "float32" else 3e-2)
+    check_each("whole", schedules.whole(engine, [request]), want, tolerances, 0.0)
+    check_each("last 60 one by one", schedules.tail_one_by_one(engine, [request], tail=60), want, tolerances, 0.0)
+    if engine.graphs is not None:
+        assert len(engine.graphs.graphs) >= 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_entry_point(folders, dtype):
     import beholdd
     folder, config, weights = folders("mixed")
