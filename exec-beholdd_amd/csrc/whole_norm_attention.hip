@@ -17,6 +17,7 @@ __global__ __launch_bounds__(256) void whole_norm_rope_write_kernel(
     const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, const int32_t* __restrict__ page_table,
     int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write) {
+  extern __shared__ float turns[];      // the cosines, then the sines, of the row's turned pairs: one of each a pair and row
   __shared__ float scratch[8];
   const int row = blockIdx.x;
   const int q_width = H * dim, k_width = G * dim, v_width = G * vdim;
@@ -24,48 +25,61 @@ __global__ __launch_bounds__(256) void whole_norm_rope_write_kernel(
   const float* k = q + q_width;
   const float* v = k + k_width;
   const int pos = positions[row];
-  float ss = 0.f;
-  for (int e = threadIdx.x; e < q_width; e += blockDim.x) ss += q[e] * q[e];
-  const float inv_q = 1.0f / sqrtf(block_sum(ss, scratch) / (float)q_width + eps);
-  for (int e = threadIdx.x; e < H * pad; e += blockDim.x) {
-    const int head = e / pad, i = e % pad;
-    float y = 0.f;
+  float* cosines = turns;
+  float* sines = turns + turned / 2;
+  for (int i = threadIdx.x; i < turned / 2; i += blockDim.x) {
+    const float angle = (float)pos * freq[i];
+    cosines[i] = cosf(angle);
+    sines[i] = sinf(angle);
+  }
+  float ss_q = 0.f, ss_k = 0.f;
+  for (int e = threadIdx.x; e < q_width + k_width; e += blockDim.x) {
+    const float x = q[e];
+    if (e < q_width) ss_q += x * x;
+    else ss_k += x * x;
+  }
+  const float inv_q = 1.0f / sqrtf(block_sum(ss_q, scratch) / (float)q_width + eps);
+  const float inv_k = 1.0f / sqrtf(block_sum(ss_k, scratch) / (float)k_width + eps);
+  // a thread takes a pair of neighbouring dimensions: both of a turned pair come from the same two loads
+  const int half = pad / 2;
+  for (int e = threadIdx.x; e < H * half; e += blockDim.x) {
+    const int head = e / half, i = 2 * (e % half);
+    float y0 = 0.f, y1 = 0.f;
     if (i < dim) {
       const int at = head * dim + i;
-      y = q[at] * inv_q * wq[at];
+      y0 = q[at] * inv_q * wq[at];
+      if (i + 1 < dim) y1 = q[at + 1] * inv_q * wq[at + 1];
       if (i < turned) {
-        const int mate = at ^ 1;
-        const float other = q[mate] * inv_q * wq[mate];
-        const float angle = (float)pos * freq[i >> 1];
-        const float c = cosf(angle), s = sinf(angle);
-        y = (i & 1) ? y * c + other * s : y * c - other * s;
+        const float c = cosines[i >> 1], s = sines[i >> 1], u = y0, w = y1;
+        y0 = u * c - w * s;
+        y1 = w * c + u * s;
       }
     }
-    q_out[(size_t)row * H * pad + e] = from_f32<T>(y);
+    T* out = q_out + (size_t)row * H * pad + head * pad + i;
+    out[0] = from_f32<T>(y0);
+    out[1] = from_f32<T>(y1);
   }
   if (!write) return;
-  ss = 0.f;
-  for (int e = threadIdx.x; e < k_width; e += blockDim.x) ss += k[e] * k[e];
-  const float inv_k = 1.0f / sqrtf(block_sum(ss, scratch) / (float)k_width + eps);
   const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE], token = pos % BH_PAGE;
-  for (int e = threadIdx.x; e < G * pad; e += blockDim.x) {
-    const int head = e / pad, i = e % pad;
-    float y = 0.f;
+  for (int e = threadIdx.x; e < G * half; e += blockDim.x) {
+    const int head = e / half, i = 2 * (e % half);
+    float y0 = 0.f, y1 = 0.f;
     if (i < dim) {
       const int at = head * dim + i;
-      y = k[at] * inv_k * wk[at];
+      y0 = k[at] * inv_k * wk[at];
+      if (i + 1 < dim) y1 = k[at + 1] * inv_k * wk[at + 1];
       if (i < turned) {
-        const int mate = at ^ 1;
-        const float other = k[mate] * inv_k * wk[mate];
-        const float angle = (float)pos * freq[i >> 1];
-        const float c = cosf(angle), s = sinf(angle);
-        y = (i & 1) ? y * c + other * s : y * c - other * s;
+        const float c = cosines[i >> 1], s = sines[i >> 1], u = y0, w = y1;
+        y0 = u * c - w * s;
+        y1 = w * c + u * s;
       }
     }
     T* keys = k_pages + ((size_t)page * G + head) * BH_PAGE * pad;
     T* values = v_pages + ((size_t)page * G + head) * BH_PAGE * pad;
-    keys[bh_key_index(kv_order, token, i, pad)] = from_f32<T>(y);
+    keys[bh_key_index(kv_order, token, i, pad)] = from_f32<T>(y0);
+    keys[bh_key_index(kv_order, token, i + 1, pad)] = from_f32<T>(y1);
     values[bh_value_index(kv_order, token, i, pad)] = from_f32<T>(i < vdim ? v[head * vdim + i] : 0.f);
+    values[bh_value_index(kv_order, token, i + 1, pad)] = from_f32<T>(i + 1 < vdim ? v[head * vdim + i + 1] : 0.f);
   }
 }
 
@@ -80,12 +94,14 @@ extern "C" int bh_whole_norm_rope_write(const float* qkv, const float* wq, const
   BH_REQUIRE(turned == 0 || freq != nullptr, "whole_norm_rope_write: a rotation needs its frequencies");
   BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && pad % 32 == 0),
              "whole_norm_rope_write: cache order %d does not exist for head size %d", kv_order, pad);
+  BH_REQUIRE(pad % 2 == 0, "whole_norm_rope_write: heads of an even size, got %d", pad);
+  const size_t lds = (size_t)(turned > 0 ? turned : 1) * sizeof(float);
   if (dtype == BH_F32)
-    whole_norm_rope_write_kernel<float><<<n_rows, 256, 0, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq, (float*)q_out,
+    whole_norm_rope_write_kernel<float><<<n_rows, 256, lds, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq, (float*)q_out,
                                                                   (float*)k_pages, (float*)v_pages, page_table, table_stride, H, G,
                                                                   dim, vdim, pad, kv_order, write);
   else if (dtype == BH_BF16)
-    whole_norm_rope_write_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq,
+    whole_norm_rope_write_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(qkv, wq, wk, eps, freq, turned, positions, row_seq,
                                                                    (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, page_table,
                                                                    table_stride, H, G, dim, vdim, pad, kv_order, write);
   else

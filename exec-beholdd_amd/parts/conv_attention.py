@@ -26,11 +26,11 @@ from .rope import RotaryFrequencies
 
 def padded_head(dim: int, vdim: int) -> int:
     """The one head size under which keys of `dim` and values of `vdim` are cached: the larger of the two, rounded up
-    to the matrix-core attention kernels' step of 32 where they take it (up to 256)."""
+    to the matrix-core attention kernels' step of 32 where they take it (up to 256), and to an even size beyond."""
     size = max(int(dim), int(vdim))
     if -(-size // 32) * 32 <= 256:
         size = -(-size // 32) * 32
-    return size
+    return size + size % 2      # the kernel that writes the heads takes their dimensions in pairs
 
 
 class ConvGatedAttention:
