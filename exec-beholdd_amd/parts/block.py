@@ -105,7 +105,6 @@ class PreNormBlock:
         self.feed_forward.forward(ctx, x, hidden)
         return None
 
-
     def _plain(self, ctx, x, hidden, cache):
         """The layer without norms that ride on products across its end: what follows the feed-forward reads the finished
         residual."""
