@@ -1068,6 +1068,7 @@ class HipKernels(KernelSizes):
             self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
 
     CONV_WALK_ROWS = 128      # from that many rows a step's convolution walks down the rows (csrc/short_conv.hip)
+    CONV_ROW_IN_LDS = 30000   # channels of q, k and v together that the one launch keeps in local memory
 
     def conv_norm_rope_write(self, proj, first, conv_weight, state, state_offset, seq_start, seq_slot, q_weight, k_weight, eps, freq,
                              turned, positions, row_seq, q_out, k_pages, v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
@@ -1076,13 +1077,15 @@ class HipKernels(KernelSizes):
         state is read, not updated (`short_conv_state` afterwards).  A step of many rows runs the two kernels after all: the
         convolution that walks down the rows loads every input once, where a workgroup per row loads it once per tap."""
         n_rows = proj.shape[0]
-        if n_rows >= self.CONV_WALK_ROWS and conv_weight is not None and 2 <= conv_weight.shape[1] <= 4:
-            conv = torch.empty((n_rows, conv_weight.shape[0]), dtype=torch.float32, device=self.device)
-            self.short_conv(proj, first, conv_weight, None, state, state_offset, row_seq, seq_start, seq_slot, conv)
+        channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
+        walks = n_rows >= self.CONV_WALK_ROWS and conv_weight is not None and 2 <= conv_weight.shape[1] <= 4
+        if walks or channels > self.CONV_ROW_IN_LDS:      # (a row of more channels does not fit the one launch's local memory)
+            weight = conv_weight if conv_weight is not None else torch.ones((channels, 1), dtype=torch.float32, device=self.device)
+            conv = torch.empty((n_rows, channels), dtype=torch.float32, device=self.device)
+            self.short_conv(proj, first, weight, None, state if weight.shape[1] > 1 else None, state_offset, row_seq, seq_start, seq_slot, conv)
             self.whole_norm_rope_write(conv, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages, v_pages, page_table,
                                        n_heads, n_kv_heads, dim, vdim, pad, write_kv)
             return
-        channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
         taps = conv_weight.shape[1] if conv_weight is not None else 0
         if tuple(q_out.shape) != (n_rows, n_heads * pad) or q_out.dtype != proj.dtype or (conv_weight is not None and conv_weight.shape[0] != channels):
             raise KernelError(f"conv_norm_rope_write: shapes proj {tuple(proj.shape)}, q_out {tuple(q_out.shape)} do not fit")
